@@ -1,0 +1,123 @@
+// C ABI of libhexa_moe_hip.so (declared in include/hexa_moe_hip.h): argument validation, dtype
+// dispatch and error reporting around the kernel launchers.  Nothing here allocates device memory
+// or waits for the device.
+#include <string.h>
+
+#include "hexa_internal.h"
+
+namespace hexa {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+static bool is_dt(int dt) { return dt == HEXA_F32 || dt == HEXA_F16 || dt == HEXA_BF16; }
+static bool is_16(int dt) { return dt == HEXA_F16 || dt == HEXA_BF16; }
+
+static int check_sizes(const char* who, int T, int k, int E, int a, int b) {
+    if (T < 0 || k < 1 || E < 1 || a < 1 || b < 1)
+        HEXA_FAIL(HEXA_ERR_ARG, "%s: bad sizes T=%d k=%d E=%d dims=(%d,%d)", who, T, k, E, a, b);
+    return HEXA_OK;
+}
+
+}  // namespace hexa
+
+using namespace hexa;
+
+extern "C" const char* hexa_last_error(void) { return g_err; }
+extern "C" int hexa_abi_version(void) { return HEXA_ABI_VERSION; }
+
+extern "C" int hexa_esmm(void* out, const void* x, const void* w, const void* bias, const int32_t* route, int m2s,
+                         int w_layout, int accumulate, int T, int k, int in_dim, int out_dim, int E, int x_dt,
+                         int w_dt, int bias_dt, int out_dt, int act, void* out_act, void* stream) {
+    if (int rc = check_sizes("hexa_esmm", T, k, E, in_dim, out_dim)) return rc;
+    if (!out || !x || !w || !route) HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: null pointer");
+    if (w_layout != HEXA_W_IN_OUT && w_layout != HEXA_W_OUT_IN) HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: bad w_layout %d", w_layout);
+    if (!is_dt(x_dt) || !is_dt(w_dt) || !is_dt(out_dt) || (bias && !is_dt(bias_dt)))
+        HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: unknown element type");
+    if (act != HEXA_ACT_NONE && act != HEXA_ACT_GELU) HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: unknown activation %d", act);
+    if (act != HEXA_ACT_NONE && (!out_act || m2s || accumulate))
+        HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: a fused activation needs out_act, m2s == 0 and accumulate == 0");
+    if (T == 0) return HEXA_OK;
+    EsmmArgs a;
+    a.out = out; a.x = x; a.w = w; a.bias = bias; a.out_act = out_act;
+    a.r = route_view(route, T, k, E);
+    a.in_dim = in_dim; a.out_dim = out_dim;
+    a.x_per_slot = m2s ? 1 : 0;
+    a.out_per_slot = m2s ? 0 : 1;
+    a.w_layout = w_layout; a.accumulate = accumulate ? 1 : 0;
+    a.x_dt = x_dt; a.w_dt = w_dt; a.bias_dt = bias_dt; a.out_dt = out_dt; a.act = act;
+    hipStream_t st = (hipStream_t)stream;
+    if (x_dt == HEXA_F32) {
+        if (w_dt != HEXA_F32 || out_dt != HEXA_F32 || (bias && bias_dt != HEXA_F32))
+            HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_esmm: fp32 tokens need fp32 weights, bias and result");
+        return launch_esmm32(a, st);
+    }
+    if (w_dt != x_dt && w_dt != HEXA_F32)
+        HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_esmm: weights must be fp32 or the tokens' 16-bit type");
+    if (out_dt != x_dt && out_dt != HEXA_F32)
+        HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_esmm: result must be fp32 or the tokens' 16-bit type");
+    if (bias && bias_dt != x_dt && bias_dt != HEXA_F32)
+        HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_esmm: bias must be fp32 or the tokens' 16-bit type");
+    return launch_esmm16(a, st);
+}
+
+extern "C" int hexa_estmm(void* dw, const void* dy, const void* x, const int32_t* route, int dy_per_slot,
+                          int x_per_slot, int accumulate, int T, int k, int out_dim, int in_dim, int E, int dt,
+                          int dw_dt, void* stream) {
+    if (int rc = check_sizes("hexa_estmm", T, k, E, in_dim, out_dim)) return rc;
+    if (!dw || !route || !dy || !x) HEXA_FAIL(HEXA_ERR_ARG, "hexa_estmm: null pointer");
+    if (!is_dt(dt) || !is_dt(dw_dt)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_estmm: unknown element type");
+    if (dw_dt != HEXA_F32 && dw_dt != dt)
+        HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_estmm: dw must be fp32 or the operands' type");
+    hipStream_t st = (hipStream_t)stream;
+    EstmmArgs a;
+    a.dw = dw; a.p = dy; a.q = x;
+    a.r = route_view(route, T, k, E);
+    a.m_dim = out_dim; a.n_dim = in_dim;
+    a.p_per_slot = dy_per_slot ? 1 : 0; a.q_per_slot = x_per_slot ? 1 : 0;
+    a.accumulate = accumulate ? 1 : 0; a.pq_dt = dt; a.dw_dt = dw_dt;
+    return is_16(dt) ? launch_estmm16(a, st) : launch_estmm32(a, st);
+}
+
+extern "C" int hexa_ess(void* db, const void* dy, const int32_t* route, int dy_per_slot, int accumulate, int T, int k,
+                        int out_dim, int E, int dt, int db_dt, void* stream) {
+    if (int rc = check_sizes("hexa_ess", T, k, E, out_dim, out_dim)) return rc;
+    if (!db || !route || !dy) HEXA_FAIL(HEXA_ERR_ARG, "hexa_ess: null pointer");
+    if (!is_dt(dt) || !is_dt(db_dt)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_ess: unknown element type");
+    hipStream_t st = (hipStream_t)stream;
+    EssArgs a;
+    a.db = db; a.dy = dy;
+    a.r = route_view(route, T, k, E);
+    a.out_dim = out_dim; a.dy_per_slot = dy_per_slot ? 1 : 0; a.accumulate = accumulate ? 1 : 0;
+    a.dy_dt = dt; a.db_dt = db_dt;
+    return launch_ess(a, st);
+}
+
+extern "C" int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y, const void* w, const void* x,
+                               const int32_t* route, int m2s, int accumulate, int T, int k, int in_dim, int out_dim,
+                               int E, int act_dt, int w_dt, int jx_dt, int jw_dt, int jb_dt, void* stream) {
+    if (!j_x || !j_w || !j_y || !w || !x || !route) HEXA_FAIL(HEXA_ERR_ARG, "hexa_fused_grad: null pointer");
+    // ESMM task: j_x = j_y . w[e] with w [E][out][in] read as an [E][in'=out][out'=in] weight; the
+    // slot layout is the mirror image of the forward's (shared j_y -> per-slot j_x and vice versa).
+    int rc = hexa_esmm(j_x, j_y, w, nullptr, route, m2s, HEXA_W_IN_OUT, accumulate, T, k, out_dim, in_dim, E, act_dt,
+                       w_dt, HEXA_F32, jx_dt, HEXA_ACT_NONE, nullptr, stream);
+    if (rc) return rc;
+    // ESTMM task: j_w[e][out][in] = sum j_y^T x
+    rc = hexa_estmm(j_w, j_y, x, route, m2s ? 1 : 0, m2s ? 0 : 1, accumulate, T, k, out_dim, in_dim, E, act_dt, jw_dt,
+                    stream);
+    if (rc) return rc;
+    if (j_b) rc = hexa_ess(j_b, j_y, route, m2s ? 1 : 0, accumulate, T, k, out_dim, E, act_dt, jb_dt, stream);
+    return rc;
+}
+
+extern "C" int hexa_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, void* stream) {
+    if (n < 0 || (n > 0 && (!dy1 || !dy2 || !y1))) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gelu_bwd: bad arguments");
+    if (!is_dt(dt)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gelu_bwd: unknown element type");
+    return launch_gelu_bwd(dy1, dy2, y1, n, dt, (hipStream_t)stream);
+}

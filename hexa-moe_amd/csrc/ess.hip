@@ -1,0 +1,163 @@
+// ESS (per-expert bias-gradient sum) and the elementwise GELU backward for gfx950.
+//
+// ESS is a gathered column sum and is bound by HBM bandwidth: one 256-thread workgroup owns one
+// (expert, strip of 8 x 16-byte columns) and streams that expert's token rows, slot after slot.  In a
+// wavefront 8 lanes cover the strip of one row and the 8 lane groups take 8 consecutive rows, so
+// every load instruction moves eight 128-byte row pieces.  fp32 partial sums stay in registers; the
+// 8 row groups of a wavefront are folded with wavefront shuffles (xor 8, 16, 32), the 4 wavefronts
+// through LDS.  Each result is written once, in a fixed order: no atomics, no zero-initialised
+// output, bit-reproducible.
+//
+// Replaces the ESS task of fused_grad_bias_kernel_vectorized_* (kernels/fused_ops_full.cu:372-431).
+#include "hexa_internal.h"
+
+namespace hexa {
+namespace {
+
+template <typename T> struct Vec16;  // 16 bytes of T
+template <> struct Vec16<float> { static constexpr int N = 4; };
+template <> struct Vec16<__bf16> { static constexpr int N = 8; };
+template <> struct Vec16<_Float16> { static constexpr int N = 8; };
+
+struct EssK {
+    const void* dy; void* db;
+    const int32_t* token_ids; const int32_t* offsets;
+    int T, k, E, N, dy_slot_rows, accumulate, db_dt;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void ess_kernel(EssK p) {
+    constexpr int V = Vec16<T>::N;
+    constexpr int STRIP = 8 * V;  // columns per workgroup
+    __shared__ float red[4][STRIP];
+    const int e = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cl = lane & 7, rg = lane >> 3;
+    const int col = blockIdx.x * STRIP + cl * V;
+    const bool col_ok = col < p.N;
+    const T* dy = reinterpret_cast<const T*>(p.dy);
+
+    float acc[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[i] = 0.f;
+
+    bool any = false;
+    for (int s = 0; s < p.k; ++s) {
+        const int beg = p.offsets[(size_t)s * (p.E + 1) + e];
+        const int end = p.offsets[(size_t)s * (p.E + 1) + e + 1];
+        any = any || end > beg;
+        const int32_t* tok = p.token_ids + (size_t)s * p.T;
+        const T* base = dy + (size_t)p.dy_slot_rows * s * p.N + col;
+        // 32 rows per workgroup step, 4 steps in flight
+        for (int r0 = beg + wave * 8 + rg; r0 < end; r0 += 128) {
+            union { uint4 u; T e[V]; } v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int r = r0 + 32 * u;
+                if (r < end && col_ok) {
+                    const int t = tok[r];
+                    v[u].u = *reinterpret_cast<const uint4*>(base + (size_t)t * p.N);
+                } else {
+                    v[u].u = make_uint4(0u, 0u, 0u, 0u);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc[i] += Cvt<T>::to_f(v[u].e[i]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+        float a = acc[i];
+        a += __shfl_xor(a, 8);
+        a += __shfl_xor(a, 16);
+        a += __shfl_xor(a, 32);
+        acc[i] = a;
+    }
+    if (rg == 0) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) red[wave][cl * V + i] = acc[i];
+    }
+    __syncthreads();
+    if (tid < STRIP) {
+        const int c = blockIdx.x * STRIP + tid;
+        if (c < p.N && (any || !p.accumulate)) {
+            const float v = red[0][tid] + red[1][tid] + red[2][tid] + red[3][tid];
+            store_out(p.db, (size_t)e * p.N + c, v, p.db_dt, p.accumulate != 0);
+        }
+    }
+}
+
+template <typename T>
+int launch_ess_t(const EssArgs& a, hipStream_t st) {
+    constexpr int STRIP = 8 * Vec16<T>::N;
+    if (a.out_dim % Vec16<T>::N)
+        HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "ess: out_dim must be a multiple of %d (got %d)", Vec16<T>::N, a.out_dim);
+    EssK p;
+    p.dy = a.dy; p.db = a.db; p.token_ids = a.r.token_ids; p.offsets = a.r.offsets;
+    p.T = a.r.T; p.k = a.r.k; p.E = a.r.E; p.N = a.out_dim;
+    p.dy_slot_rows = a.dy_per_slot ? a.r.T : 0;
+    p.accumulate = a.accumulate; p.db_dt = a.db_dt;
+    dim3 grid(div_up(a.out_dim, STRIP), a.r.E);
+    hipLaunchKernelGGL((ess_kernel<T>), grid, dim3(256), 0, st, p);
+    HEXA_CHECK_LAUNCH("ess");
+    return HEXA_OK;
+}
+
+// dy1 = dy2 * gelu'(y1),  gelu'(x) = Phi(x) + x * phi(x)
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_bwd_kernel(T* __restrict__ dy1, const T* __restrict__ dy2,
+                                                       const T* __restrict__ y1, int64_t n) {
+    constexpr int V = Vec16<T>::N;
+    const int64_t nv = n / V;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nv; i += stride) {
+        union { uint4 u; T e[V]; } g, y, o;
+        g.u = reinterpret_cast<const uint4*>(dy2)[i];
+        y.u = reinterpret_cast<const uint4*>(y1)[i];
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            const float x = Cvt<T>::to_f(y.e[j]);
+            const float cdf = 0.5f * (1.0f + erff(x * 0.70710678118654752440f));
+            const float pdf = 0.39894228040143267794f * __expf(-0.5f * x * x);
+            o.e[j] = Cvt<T>::from_f(Cvt<T>::to_f(g.e[j]) * (cdf + x * pdf));
+        }
+        reinterpret_cast<uint4*>(dy1)[i] = o.u;
+    }
+    // tail (n not a multiple of the vector width)
+    for (int64_t i = nv * V + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const float x = Cvt<T>::to_f(y1[i]);
+        const float cdf = 0.5f * (1.0f + erff(x * 0.70710678118654752440f));
+        const float pdf = 0.39894228040143267794f * __expf(-0.5f * x * x);
+        dy1[i] = Cvt<T>::from_f(Cvt<T>::to_f(dy2[i]) * (cdf + x * pdf));
+    }
+}
+
+template <typename T>
+int launch_gelu_bwd_t(void* dy1, const void* dy2, const void* y1, int64_t n, hipStream_t st) {
+    if (n == 0) return HEXA_OK;
+    int64_t blocks = (n / Vec16<T>::N + 255) / 256;
+    if (blocks < 1) blocks = 1;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    hipLaunchKernelGGL((gelu_bwd_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, (T*)dy1, (const T*)dy2,
+                       (const T*)y1, n);
+    HEXA_CHECK_LAUNCH("gelu_bwd");
+    return HEXA_OK;
+}
+
+}  // namespace
+
+int launch_ess(const EssArgs& a, hipStream_t st) {
+    if (a.dy_dt == HEXA_F32) return launch_ess_t<float>(a, st);
+    if (a.dy_dt == HEXA_BF16) return launch_ess_t<__bf16>(a, st);
+    return launch_ess_t<_Float16>(a, st);
+}
+
+int launch_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, hipStream_t st) {
+    if (dt == HEXA_F32) return launch_gelu_bwd_t<float>(dy1, dy2, y1, n, st);
+    if (dt == HEXA_BF16) return launch_gelu_bwd_t<__bf16>(dy1, dy2, y1, n, st);
+    return launch_gelu_bwd_t<_Float16>(dy1, dy2, y1, n, st);
+}
+
+}  // namespace hexa

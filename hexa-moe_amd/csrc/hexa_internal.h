@@ -1,0 +1,117 @@
+// Internal declarations shared by the HIP translation units of libhexa_moe_hip.so.
+// The public C ABI is include/hexa_moe_hip.h; nothing here is exported.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/hexa_moe_hip.h"
+
+namespace hexa {
+
+// ---- error plumbing -----------------------------------------------------------------------
+void set_error(const char* fmt, ...);
+
+#define HEXA_FAIL(code, ...)                \
+    do {                                    \
+        ::hexa::set_error(__VA_ARGS__);     \
+        return (code);                      \
+    } while (0)
+
+#define HEXA_CHECK_LAUNCH(what)                                                        \
+    do {                                                                               \
+        hipError_t e__ = hipGetLastError();                                            \
+        if (e__ != hipSuccess) HEXA_FAIL(HEXA_ERR_LAUNCH, "%s: launch failed: %s", what, \
+                                         hipGetErrorString(e__));                      \
+    } while (0)
+
+// ---- tiling constants shared between the routing pass and the matmul kernels ----------------
+// Row tile of the gathered-row grouped GEMM (ESMM).  The routing pass emits one tile_info entry
+// per HEXA_TILE_ROWS rows of every (slot, expert) segment.
+constexpr int kTileRows = HEXA_TILE_ROWS;
+
+static inline int div_up(int a, int b) { return (a + b - 1) / b; }
+
+// ---- routing metadata view (all device pointers) --------------------------------------------
+struct RouteView {
+    const int32_t* token_ids;   // [k][list_stride]
+    const int32_t* offsets;     // [k][E+1]
+    const int4* tile_info;      // [k][mt_ub]: {expert, row_start, row_count, 0}
+    const int32_t* tile_count;  // [k]
+    int T, k, E, mt_ub;
+};
+
+RouteView route_view(const int32_t* route, int T, int k, int E);
+
+// ---- launchers implemented in the kernel files ----------------------------------------------
+struct EsmmArgs {
+    void* out; const void* x; const void* w; const void* bias; void* out_act;
+    RouteView r;
+    int in_dim, out_dim;
+    int x_per_slot, out_per_slot;  // row operand / result indexed [slot][T][*] (1) or [T][*] (0)
+    int w_layout;                  // HEXA_W_IN_OUT: [E][in][out]; HEXA_W_OUT_IN: [E][out][in]
+    int accumulate;                // result += instead of =
+    int x_dt, w_dt, bias_dt, out_dt;
+    int act;
+};
+struct EstmmArgs {
+    void* dw; const void* p; const void* q;   // dw[e][m][n] = sum_rows p[row][m] * q[row][n]
+    RouteView r;
+    int m_dim, n_dim;
+    int p_per_slot, q_per_slot;
+    int accumulate;
+    int pq_dt, dw_dt;
+};
+struct EssArgs {
+    void* db; const void* dy;
+    RouteView r;
+    int out_dim, dy_per_slot, accumulate, dy_dt, db_dt;
+};
+
+int launch_esmm16(const EsmmArgs& a, hipStream_t s);
+int launch_esmm32(const EsmmArgs& a, hipStream_t s);
+int launch_estmm16(const EstmmArgs& a, hipStream_t s);
+int launch_estmm32(const EstmmArgs& a, hipStream_t s);
+int launch_ess(const EssArgs& a, hipStream_t s);
+int launch_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, hipStream_t s);
+
+// ---- small device helpers -------------------------------------------------------------------
+__device__ __forceinline__ float gelu_erf(float x) {
+    return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+}
+
+template <typename T> struct Cvt;
+template <> struct Cvt<float> {
+    static __device__ __forceinline__ float to_f(float v) { return v; }
+    static __device__ __forceinline__ float from_f(float v) { return v; }
+};
+template <> struct Cvt<__bf16> {
+    static __device__ __forceinline__ float to_f(__bf16 v) { return (float)v; }
+    static __device__ __forceinline__ __bf16 from_f(float v) { return (__bf16)v; }
+};
+template <> struct Cvt<_Float16> {
+    static __device__ __forceinline__ float to_f(_Float16 v) { return (float)v; }
+    static __device__ __forceinline__ _Float16 from_f(float v) { return (_Float16)v; }
+};
+
+// Store / accumulate one fp32 value into a result buffer whose element type is chosen at run time.
+__device__ __forceinline__ void store_out(void* base, size_t idx, float v, int dt, bool accumulate) {
+    if (dt == HEXA_F32) {
+        float* p = (float*)base + idx;
+        *p = accumulate ? (*p + v) : v;
+    } else if (dt == HEXA_BF16) {
+        __bf16* p = (__bf16*)base + idx;
+        *p = (__bf16)(accumulate ? ((float)*p + v) : v);
+    } else {
+        _Float16* p = (_Float16*)base + idx;
+        *p = (_Float16)(accumulate ? ((float)*p + v) : v);
+    }
+}
+__device__ __forceinline__ float load_as_f(const void* base, size_t idx, int dt) {
+    if (dt == HEXA_F32) return ((const float*)base)[idx];
+    if (dt == HEXA_BF16) return (float)((const __bf16*)base)[idx];
+    return (float)((const _Float16*)base)[idx];
+}
+
+}  // namespace hexa

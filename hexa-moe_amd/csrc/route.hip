@@ -1,0 +1,354 @@
+// Routing segment pass for gfx950: per-expert token lists without padding, dropping or host sync.
+//
+// Three small launches over (wavefront unit, slot):
+//   1. route_hist    one wavefront per HEXA_ROUTE_UNIT consecutive tokens: LDS histogram
+//   2. route_scan    one workgroup per slot: per-expert exclusive prefix over the units, exclusive
+//                    scan over experts (wavefront shuffles), row-tile records for the matmul kernels
+//   3. route_scatter one wavefront per unit again: stable rank of every token inside its
+//                    (unit, expert) group from log2(E) ballots, so a segment lists its tokens in
+//                    ascending order -- the result is a stable counting sort and is bit-reproducible.
+// Replaces launch_count / launch_assign of the reference (kernels/shared_cuda_core.cu:126-182,
+// 284-333), which run single-workgroup launches with shared-memory atomics, two blocking copies and
+// a host-side prefix per call.
+#include "hexa_internal.h"
+
+namespace hexa {
+namespace {
+
+constexpr int kUnit = HEXA_ROUTE_UNIT;
+constexpr int kWave = 64;
+
+template <typename IdxT>
+__global__ __launch_bounds__(kWave) void route_hist_kernel(const IdxT* __restrict__ routing,
+                                                           int64_t token_stride, int64_t slot_stride,
+                                                           int T, int E, int units,
+                                                           int32_t* __restrict__ unit_hist) {
+    extern __shared__ int32_t sh[];
+    const int lane = threadIdx.x, unit = blockIdx.x, s = blockIdx.y;
+    for (int i = lane; i < E; i += kWave) sh[i] = 0;
+    __syncthreads();
+    const int t0 = unit * kUnit;
+    const int t1 = min(T, t0 + kUnit);
+    for (int t = t0 + lane; t < t1; t += kWave) {
+        long e = (long)routing[(int64_t)t * token_stride + (int64_t)s * slot_stride];
+        if (e >= 0 && e < E) atomicAdd(&sh[e], 1);
+    }
+    __syncthreads();
+    int32_t* dst = unit_hist + ((size_t)s * units + unit) * E;
+    for (int i = lane; i < E; i += kWave) dst[i] = sh[i];
+}
+
+// Exclusive scan of one int per thread over a 256-thread workgroup; returns the exclusive prefix
+// and the workgroup total.  tmp: 8 ints of LDS.
+__device__ __forceinline__ int block_excl_scan_256(int v, int* tmp, int& total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        int o = __shfl_up(incl, d);
+        if (lane >= d) incl += o;
+    }
+    if (lane == 63) tmp[wave] = incl;
+    __syncthreads();
+    int base = 0;
+    for (int w = 0; w < wave; ++w) base += tmp[w];
+    total = tmp[0] + tmp[1] + tmp[2] + tmp[3];
+    __syncthreads();
+    return base + incl - v;
+}
+
+// Given per-expert totals in LDS (tot[E]), write counts / offsets (exclusive prefix of the totals
+// rounded up to `pad`) and, when tile_info != nullptr, one record per kTileRows rows of each
+// segment.  LDS: tot[E], off[E+1], tbase[E+1], tmp[8].
+__device__ void finish_slot(const int32_t* tot, int32_t* off, int32_t* tbase, int* tmp, int E, int pad,
+                            int32_t* counts, int32_t* offsets, int4* tile_info, int32_t* tile_count,
+                            int mt_ub) {
+    const int tid = threadIdx.x;
+    const int chunk = (E + 255) / 256;
+    const int e0 = min(E, tid * chunk), e1 = min(E, e0 + chunk);
+    int sum_rows = 0, sum_tiles = 0;
+    for (int e = e0; e < e1; ++e) {
+        int c = tot[e];
+        sum_rows += ((c + pad - 1) / pad) * pad;
+        sum_tiles += (c + kTileRows - 1) / kTileRows;
+    }
+    int total_rows, total_tiles;
+    int row_base = block_excl_scan_256(sum_rows, tmp, total_rows);
+    int tile_base = block_excl_scan_256(sum_tiles, tmp, total_tiles);
+    for (int e = e0; e < e1; ++e) {
+        int c = tot[e];
+        off[e] = row_base;
+        tbase[e] = tile_base;
+        row_base += ((c + pad - 1) / pad) * pad;
+        tile_base += (c + kTileRows - 1) / kTileRows;
+    }
+    if (tid == 0) { off[E] = total_rows; tbase[E] = total_tiles; }
+    __syncthreads();
+    for (int e = tid; e <= E; e += 256) {
+        if (offsets) offsets[e] = off[e];
+        if (counts && e < E) counts[e] = tot[e];
+    }
+    if (tile_info) {
+        if (tid == 0) *tile_count = total_tiles;
+        const int n = min(total_tiles, mt_ub);
+        for (int m = tid; m < n; m += 256) {
+            // last expert whose first tile index is <= m (experts without tiles share a base)
+            int lo = 0, hi = E;  // invariant: tbase[lo] <= m < tbase[hi]
+            while (hi - lo > 1) {
+                int mid = (lo + hi) >> 1;
+                if (tbase[mid] <= m) lo = mid; else hi = mid;
+            }
+            int j = m - tbase[lo];
+            int rows = min(kTileRows, tot[lo] - j * kTileRows);
+            tile_info[m] = make_int4(lo, off[lo] + j * kTileRows, rows, 0);
+        }
+    }
+}
+
+// One workgroup per slot.  Turns unit_hist[s][u][e] into the exclusive prefix over u (in place) and
+// finishes the slot.  given_offsets != nullptr: legacy TOKEN_ASSIGN, segment starts come from the
+// caller and nothing but the unit prefixes is written.
+__global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ unit_hist, int E, int units,
+                                                         int pad, int32_t* __restrict__ counts,
+                                                         int32_t* __restrict__ offsets,
+                                                         int4* __restrict__ tile_info,
+                                                         int32_t* __restrict__ tile_count, int mt_ub,
+                                                         int prefix_only) {
+    extern __shared__ int32_t sh[];
+    int32_t* tot = sh;
+    int32_t* off = tot + E;
+    int32_t* tbase = off + (E + 1);
+    int* tmp = tbase + (E + 1);
+    const int s = blockIdx.x;
+    int32_t* H = unit_hist + (size_t)s * units * E;
+    for (int e = threadIdx.x; e < E; e += 256) {
+        int run = 0;
+        for (int u = 0; u < units; ++u) {
+            int c = H[(size_t)u * E + e];
+            H[(size_t)u * E + e] = run;
+            run += c;
+        }
+        tot[e] = run;
+    }
+    __syncthreads();
+    if (prefix_only) return;
+    finish_slot(tot, off, tbase, tmp, E, pad, counts ? counts + (size_t)s * E : nullptr,
+                offsets ? offsets + (size_t)s * (E + 1) : nullptr,
+                tile_info ? tile_info + (size_t)s * mt_ub : nullptr, tile_count ? tile_count + s : nullptr,
+                mt_ub);
+}
+
+template <typename IdxT>
+__global__ __launch_bounds__(kWave) void route_scatter_kernel(const IdxT* __restrict__ routing,
+                                                              int64_t token_stride, int64_t slot_stride,
+                                                              int T, int E, int units, int nbits,
+                                                              const int32_t* __restrict__ unit_hist,
+                                                              const int32_t* __restrict__ offsets,
+                                                              int64_t offsets_slot_stride,
+                                                              int32_t* __restrict__ token_ids,
+                                                              int32_t* __restrict__ expert_ids,
+                                                              int64_t list_stride) {
+    extern __shared__ int32_t cursor[];
+    const int lane = threadIdx.x, unit = blockIdx.x, s = blockIdx.y;
+    const int32_t* H = unit_hist + ((size_t)s * units + unit) * E;
+    const int32_t* off = offsets + (size_t)s * offsets_slot_stride;
+    for (int i = lane; i < E; i += kWave) cursor[i] = off[i] + H[i];
+    __syncthreads();
+    const int t0 = unit * kUnit;
+    const int t1 = min(T, t0 + kUnit);
+    const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    int32_t* tok = token_ids + (size_t)s * list_stride;
+    int32_t* exp = expert_ids ? expert_ids + (size_t)s * list_stride : nullptr;
+    for (int base = t0; base < t1; base += kWave) {   // trip count is uniform over the wavefront
+        const int t = base + lane;
+        long e = -1;
+        if (t < t1) e = (long)routing[(int64_t)t * token_stride + (int64_t)s * slot_stride];
+        const bool valid = (e >= 0 && e < E);
+        // lanes holding the same expert id: AND over the id's bits of "lanes that agree on the bit"
+        unsigned long long peers = __ballot(valid);
+        for (int b = 0; b < nbits; ++b) {
+            const bool bit = (e >> b) & 1;
+            const unsigned long long m = __ballot(valid && bit);
+            peers &= bit ? m : ~m;
+        }
+        int pos = 0;
+        if (valid) pos = cursor[e] + __popcll(peers & lt_mask);
+        __syncthreads();
+        if (valid) {
+            tok[pos] = t;
+            if (exp) exp[pos] = (int32_t)e;
+            if ((peers & lt_mask) == 0) cursor[e] += __popcll(peers);  // first lane of its group
+        }
+        __syncthreads();
+    }
+}
+
+// offsets from a list sorted by expert: lower bounds by binary search, then the same finish.
+__global__ __launch_bounds__(256) void route_from_lists_kernel(const int32_t* __restrict__ expert_idx_list,
+                                                               int T, int E, int32_t* __restrict__ counts,
+                                                               int32_t* __restrict__ offsets,
+                                                               int4* __restrict__ tile_info,
+                                                               int32_t* __restrict__ tile_count, int mt_ub) {
+    extern __shared__ int32_t sh[];
+    int32_t* tot = sh;
+    int32_t* off = tot + E;
+    int32_t* tbase = off + (E + 1);
+    int* tmp = tbase + (E + 1);
+    const int s = blockIdx.x;
+    const int32_t* L = expert_idx_list + (size_t)s * T;
+    for (int e = threadIdx.x; e < E; e += 256) {
+        int lo = 0, hi = T;  // first position with L[pos] >= e
+        while (lo < hi) { int mid = (lo + hi) >> 1; if (L[mid] < e) lo = mid + 1; else hi = mid; }
+        int lb = lo;
+        lo = lb; hi = T;     // first position with L[pos] > e
+        while (lo < hi) { int mid = (lo + hi) >> 1; if (L[mid] <= e) lo = mid + 1; else hi = mid; }
+        tot[e] = lo - lb;
+    }
+    __syncthreads();
+    finish_slot(tot, off, tbase, tmp, E, 1, counts + (size_t)s * E, offsets + (size_t)s * (E + 1),
+                tile_info + (size_t)s * mt_ub, tile_count + s, mt_ub);
+}
+
+int ceil_log2(int n) { int b = 0; while ((1 << b) < n) ++b; return b; }
+
+size_t scan_lds_bytes(int E) { return sizeof(int32_t) * (size_t)(E + 2 * (E + 1) + 8); }
+
+}  // namespace
+}  // namespace hexa
+
+using namespace hexa;
+
+extern "C" int hexa_route_layout_get(int T, int k, int E, hexa_route_layout* out) {
+    if (!out) HEXA_FAIL(HEXA_ERR_ARG, "hexa_route_layout_get: null layout");
+    if (T < 0 || k < 1 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_route_layout_get: bad sizes T=%d k=%d E=%d", T, k, E);
+    const int64_t K = k;
+    out->mt_ub = T / HEXA_TILE_ROWS + E;
+    out->units = T > 0 ? div_up(T, HEXA_ROUTE_UNIT) : 1;
+    int64_t p = 0;
+    out->counts = p;      p += K * E;
+    out->offsets = p;     p += K * (E + 1);
+    out->token_ids = p;   p += K * T;
+    out->expert_ids = p;  p += K * T;
+    out->tile_count = p;  p += K;
+    p = (p + 3) & ~(int64_t)3;  // tile records are 16-byte vectors
+    out->tile_info = p;   p += K * out->mt_ub * 4;
+    out->scratch = p;     p += K * out->units * E;
+    out->total_ints = p;
+    return HEXA_OK;
+}
+
+namespace hexa {
+RouteView route_view(const int32_t* route, int T, int k, int E) {
+    hexa_route_layout L;
+    hexa_route_layout_get(T, k, E, &L);
+    RouteView v;
+    v.token_ids = route + L.token_ids;
+    v.offsets = route + L.offsets;
+    v.tile_info = reinterpret_cast<const int4*>(route + L.tile_info);
+    v.tile_count = route + L.tile_count;
+    v.T = T; v.k = k; v.E = E; v.mt_ub = L.mt_ub;
+    return v;
+}
+}  // namespace hexa
+
+static int check_route_sizes(const char* who, int T, int k, int E) {
+    if (T < 0 || k < 1 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "%s: bad sizes T=%d k=%d E=%d", who, T, k, E);
+    if (E > 8192) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "%s: more than 8192 experts (E=%d)", who, E);
+    return HEXA_OK;
+}
+
+extern "C" int hexa_route_build(const void* routing, int routing_is_i64, int64_t token_stride, int64_t slot_stride,
+                                int T, int k, int E, int32_t* route, void* stream) {
+    if (int rc = check_route_sizes("hexa_route_build", T, k, E)) return rc;
+    if (!route || (T > 0 && !routing)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_route_build: null pointer");
+    if (((uintptr_t)route & 15) != 0) HEXA_FAIL(HEXA_ERR_ARG, "hexa_route_build: route blob must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    hexa_route_layout L;
+    hexa_route_layout_get(T, k, E, &L);
+    int32_t* H = route + L.scratch;
+    dim3 grid(L.units, k);
+    if (routing_is_i64)
+        hipLaunchKernelGGL(route_hist_kernel<int64_t>, grid, dim3(kWave), sizeof(int32_t) * E, st,
+                           (const int64_t*)routing, token_stride, slot_stride, T, E, L.units, H);
+    else
+        hipLaunchKernelGGL(route_hist_kernel<int32_t>, grid, dim3(kWave), sizeof(int32_t) * E, st,
+                           (const int32_t*)routing, token_stride, slot_stride, T, E, L.units, H);
+    HEXA_CHECK_LAUNCH("route_hist");
+    hipLaunchKernelGGL(route_scan_kernel, dim3(k), dim3(256), scan_lds_bytes(E), st, H, E, L.units, 1,
+                       route + L.counts, route + L.offsets, reinterpret_cast<int4*>(route + L.tile_info),
+                       route + L.tile_count, L.mt_ub, 0);
+    HEXA_CHECK_LAUNCH("route_scan");
+    const int nbits = ceil_log2(E);
+    if (routing_is_i64)
+        hipLaunchKernelGGL(route_scatter_kernel<int64_t>, grid, dim3(kWave), sizeof(int32_t) * E, st,
+                           (const int64_t*)routing, token_stride, slot_stride, T, E, L.units, nbits, H,
+                           route + L.offsets, (int64_t)(E + 1), route + L.token_ids, route + L.expert_ids,
+                           (int64_t)T);
+    else
+        hipLaunchKernelGGL(route_scatter_kernel<int32_t>, grid, dim3(kWave), sizeof(int32_t) * E, st,
+                           (const int32_t*)routing, token_stride, slot_stride, T, E, L.units, nbits, H,
+                           route + L.offsets, (int64_t)(E + 1), route + L.token_ids, route + L.expert_ids,
+                           (int64_t)T);
+    HEXA_CHECK_LAUNCH("route_scatter");
+    return HEXA_OK;
+}
+
+extern "C" int hexa_token_count(int32_t* tokens_per_expert, int32_t* expanded, const int32_t* routing, int T, int E,
+                                int pad, int32_t* scratch, void* stream) {
+    if (int rc = check_route_sizes("hexa_token_count", T, 1, E)) return rc;
+    if (!tokens_per_expert || !expanded || !scratch || (T > 0 && !routing))
+        HEXA_FAIL(HEXA_ERR_ARG, "hexa_token_count: null pointer");
+    if (pad < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_token_count: pad must be >= 1 (got %d)", pad);
+    hipStream_t st = (hipStream_t)stream;
+    const int units = T > 0 ? div_up(T, HEXA_ROUTE_UNIT) : 1;
+    hipLaunchKernelGGL(route_hist_kernel<int32_t>, dim3(units, 1), dim3(kWave), sizeof(int32_t) * E, st, routing,
+                       (int64_t)1, (int64_t)0, T, E, units, scratch);
+    HEXA_CHECK_LAUNCH("route_hist");
+    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(256), scan_lds_bytes(E), st, scratch, E, units, pad,
+                       tokens_per_expert, expanded, (int4*)nullptr, (int32_t*)nullptr, 0, 0);
+    HEXA_CHECK_LAUNCH("route_scan");
+    return HEXA_OK;
+}
+
+extern "C" int hexa_token_assign(int32_t* token_idx_list, int32_t* expert_idx_list, const int32_t* expanded,
+                                 const int32_t* routing, int T, int E, int32_t* scratch, void* stream) {
+    if (int rc = check_route_sizes("hexa_token_assign", T, 1, E)) return rc;
+    if (!token_idx_list || !expert_idx_list || !expanded || !scratch || (T > 0 && !routing))
+        HEXA_FAIL(HEXA_ERR_ARG, "hexa_token_assign: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const int units = T > 0 ? div_up(T, HEXA_ROUTE_UNIT) : 1;
+    hipLaunchKernelGGL(route_hist_kernel<int32_t>, dim3(units, 1), dim3(kWave), sizeof(int32_t) * E, st, routing,
+                       (int64_t)1, (int64_t)0, T, E, units, scratch);
+    HEXA_CHECK_LAUNCH("route_hist");
+    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(256), scan_lds_bytes(E), st, scratch, E, units, 1,
+                       (int32_t*)nullptr, (int32_t*)nullptr, (int4*)nullptr, (int32_t*)nullptr, 0, 1);
+    HEXA_CHECK_LAUNCH("route_scan");
+    hipLaunchKernelGGL(route_scatter_kernel<int32_t>, dim3(units, 1), dim3(kWave), sizeof(int32_t) * E, st, routing,
+                       (int64_t)1, (int64_t)0, T, E, units, ceil_log2(E), scratch, expanded, (int64_t)0,
+                       token_idx_list, expert_idx_list, (int64_t)0);
+    HEXA_CHECK_LAUNCH("route_scatter");
+    return HEXA_OK;
+}
+
+extern "C" int hexa_route_from_lists(const int32_t* token_idx_list, const int32_t* expert_idx_list, int T, int k,
+                                     int E, int32_t* route, void* stream) {
+    if (int rc = check_route_sizes("hexa_route_from_lists", T, k, E)) return rc;
+    if (!route || (T > 0 && (!token_idx_list || !expert_idx_list)))
+        HEXA_FAIL(HEXA_ERR_ARG, "hexa_route_from_lists: null pointer");
+    if (((uintptr_t)route & 15) != 0) HEXA_FAIL(HEXA_ERR_ARG, "hexa_route_from_lists: route blob must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    hexa_route_layout L;
+    hexa_route_layout_get(T, k, E, &L);
+    if (T > 0) {
+        hipError_t e1 = hipMemcpyAsync(route + L.token_ids, token_idx_list, sizeof(int32_t) * (size_t)k * T,
+                                       hipMemcpyDeviceToDevice, st);
+        hipError_t e2 = hipMemcpyAsync(route + L.expert_ids, expert_idx_list, sizeof(int32_t) * (size_t)k * T,
+                                       hipMemcpyDeviceToDevice, st);
+        if (e1 != hipSuccess || e2 != hipSuccess) HEXA_FAIL(HEXA_ERR_LAUNCH, "hexa_route_from_lists: copy failed");
+    }
+    hipLaunchKernelGGL(route_from_lists_kernel, dim3(k), dim3(256), scan_lds_bytes(E), st, expert_idx_list, T, E,
+                       route + L.counts, route + L.offsets, reinterpret_cast<int4*>(route + L.tile_info),
+                       route + L.tile_count, L.mt_ub);
+    HEXA_CHECK_LAUNCH("route_from_lists");
+    return HEXA_OK;
+}

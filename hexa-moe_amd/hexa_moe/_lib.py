@@ -1,0 +1,75 @@
+"""ctypes binding of libhexa_moe_hip.so (the C ABI in include/hexa_moe_hip.h).
+
+The library is built in-tree by `make -C hexa-moe_amd/csrc` (or __graft_entry__.build()).  There is
+no fallback: if it is missing, or an entry point returns an error code, a RuntimeError is raised.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "lib", "libhexa_moe_hip.so"))
+
+HEXA_F32, HEXA_F16, HEXA_BF16 = 0, 1, 2
+HEXA_W_IN_OUT, HEXA_W_OUT_IN = 0, 1
+HEXA_ACT_NONE, HEXA_ACT_GELU = 0, 1
+HEXA_TILE_ROWS = 128
+HEXA_ROUTE_UNIT = 512
+
+_vp, _i, _i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
+
+
+class RouteLayout(ctypes.Structure):
+    _fields_ = [("counts", _i64), ("offsets", _i64), ("token_ids", _i64), ("expert_ids", _i64),
+                ("tile_count", _i64), ("tile_info", _i64), ("scratch", _i64), ("total_ints", _i64),
+                ("mt_ub", ctypes.c_int32), ("units", ctypes.c_int32)]
+
+
+# name -> (restype, argtypes); kept in one table so the export test can walk it
+SIGNATURES = {
+    "hexa_route_layout_get": (_i, [_i, _i, _i, ctypes.POINTER(RouteLayout)]),
+    "hexa_route_build": (_i, [_vp, _i, _i64, _i64, _i, _i, _i, _vp, _vp]),
+    "hexa_token_count": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
+    "hexa_token_assign": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
+    "hexa_route_from_lists": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
+    "hexa_esmm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
+    "hexa_estmm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "hexa_ess": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "hexa_fused_grad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "hexa_gelu_bwd": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),
+    "hexa_last_error": (ctypes.c_char_p, []),
+    "hexa_abi_version": (_i, []),
+}
+
+_lib = None
+
+
+def load():
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"hexa_moe: {LIB_PATH} is missing. Build it with `make -C hexa-moe_amd/csrc` "
+            "(hipcc, gfx950). There is no fallback implementation.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    if lib.hexa_abi_version() != 1:
+        raise RuntimeError("hexa_moe: libhexa_moe_hip.so has an unexpected ABI version")
+    _lib = lib
+    return lib
+
+
+def check(rc, what):
+    if rc != 0:
+        msg = load().hexa_last_error()
+        raise RuntimeError(f"{what} failed (code {rc}): {msg.decode() if msg else ''}")
+
+
+def route_layout(T, k, E):
+    L = RouteLayout()
+    check(load().hexa_route_layout_get(int(T), int(k), int(E), ctypes.byref(L)), "hexa_route_layout_get")
+    return L

@@ -1,0 +1,185 @@
+"""Tensor-level wrappers of the C ABI: device memory and streams come from PyTorch, everything else
+happens in libhexa_moe_hip.so.  All tensors must live on a HIP device; CPU tensors are rejected."""
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: _lib.HEXA_F32, torch.float16: _lib.HEXA_F16, torch.bfloat16: _lib.HEXA_BF16}
+
+
+def _dt(t):
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise TypeError(f"hexa_moe: unsupported element type {t.dtype}")
+
+
+def _dev(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("hexa_moe: expert-specific operators run on the GPU only; got a CPU tensor "
+                               "(there is no CPU fallback)")
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+class Route:
+    """Routing metadata of one MoE depth: a view of a caller-owned int32 blob (see
+    hexa_route_layout in include/hexa_moe_hip.h)."""
+
+    def __init__(self, blob, T, k, E):
+        self.blob, self.T, self.k, self.E = blob, int(T), int(k), int(E)
+        self.layout = _lib.route_layout(T, k, E)
+
+    def _part(self, start, n):
+        return self.blob[start:start + n]
+
+    @property
+    def counts(self):
+        return self._part(self.layout.counts, self.k * self.E).view(self.k, self.E)
+
+    @property
+    def offsets(self):
+        return self._part(self.layout.offsets, self.k * (self.E + 1)).view(self.k, self.E + 1)
+
+    @property
+    def token_ids(self):
+        return self._part(self.layout.token_ids, self.k * self.T).view(self.k, self.T)
+
+    @property
+    def expert_ids(self):
+        return self._part(self.layout.expert_ids, self.k * self.T).view(self.k, self.T)
+
+    @property
+    def tile_count(self):
+        return self._part(self.layout.tile_count, self.k)
+
+    @property
+    def tile_info(self):
+        return self._part(self.layout.tile_info, self.k * self.layout.mt_ub * 4).view(self.k, self.layout.mt_ub, 4)
+
+
+class RouteWorkspace:
+    """One int32 device buffer reused by every MoE depth of a model (the depth-shared cache of
+    routing metadata).  It grows to the largest (T, k, E) seen and is never shrunk."""
+
+    def __init__(self):
+        self.buf = None
+
+    def get(self, T, k, E, device):
+        need = _lib.route_layout(T, k, E).total_ints
+        if self.buf is None or self.buf.numel() < need or self.buf.device != device:
+            self.buf = torch.empty(max(int(need), 4), dtype=torch.int32, device=device)
+        return self.buf
+
+
+def route_blob_ints(T, k, E):
+    return int(_lib.route_layout(T, k, E).total_ints)
+
+
+def route_build(routing, num_experts, blob=None):
+    """routing: [T, k] (or [T]) int32/int64 expert choices on the GPU -> Route."""
+    _dev(routing)
+    if routing.dim() == 1:
+        routing = routing.unsqueeze(1)
+    if routing.dtype not in (torch.int32, torch.int64):
+        raise TypeError("hexa_moe: routing must be int32 or int64")
+    T, k = routing.shape
+    if blob is None:
+        blob = torch.empty(max(route_blob_ints(T, k, num_experts), 4), dtype=torch.int32, device=routing.device)
+    rc = _lib.load().hexa_route_build(_ptr(routing), int(routing.dtype == torch.int64), routing.stride(0),
+                                      routing.stride(1), T, k, num_experts, _ptr(blob), _stream())
+    _lib.check(rc, "hexa_route_build")
+    return Route(blob, T, k, num_experts)
+
+
+def route_from_lists(token_idx_list, expert_idx_list, T, k, num_experts, blob=None):
+    _dev(token_idx_list, expert_idx_list)
+    if blob is None:
+        blob = torch.empty(max(route_blob_ints(T, k, num_experts), 4), dtype=torch.int32, device=token_idx_list.device)
+    rc = _lib.load().hexa_route_from_lists(_ptr(token_idx_list), _ptr(expert_idx_list), T, k, num_experts,
+                                           _ptr(blob), _stream())
+    _lib.check(rc, "hexa_route_from_lists")
+    return Route(blob, T, k, num_experts)
+
+
+def esmm(x, w, bias, route, m2s, w_layout, out=None, out_dtype=None, accumulate=False, gelu=False):
+    """out[(s),t] (+)= x[(s),t] @ W[e] + bias[e].  Returns out, or (out, gelu(out)) when gelu=True."""
+    _dev(x, w, bias, out)
+    T, k, E = route.T, route.k, route.E
+    x = x.contiguous()
+    w = w.contiguous()
+    if w_layout == _lib.HEXA_W_IN_OUT:
+        in_dim, out_dim = w.shape[1], w.shape[2]
+    else:
+        out_dim, in_dim = w.shape[1], w.shape[2]
+    assert w.shape[0] == E and x.shape[-1] == in_dim
+    assert tuple(x.shape) == ((k, T, in_dim) if m2s else (T, in_dim)), (x.shape, m2s, k, T, in_dim)
+    if out is None:
+        assert not accumulate
+        out_dtype = out_dtype or x.dtype
+        out = torch.empty((T, out_dim) if m2s else (k, T, out_dim), dtype=out_dtype, device=x.device)
+    assert out.is_contiguous() and tuple(out.shape) == ((T, out_dim) if m2s else (k, T, out_dim))
+    out_act = torch.empty_like(out) if gelu else None
+    if bias is not None:
+        bias = bias.contiguous()
+    rc = _lib.load().hexa_esmm(_ptr(out), _ptr(x), _ptr(w), _ptr(bias), _ptr(route.blob), int(bool(m2s)),
+                               int(w_layout), int(bool(accumulate)), T, k, in_dim, out_dim, E, _dt(x), _dt(w),
+                               _dt(bias) if bias is not None else 0, _dt(out),
+                               _lib.HEXA_ACT_GELU if gelu else _lib.HEXA_ACT_NONE, _ptr(out_act), _stream())
+    _lib.check(rc, "hexa_esmm")
+    return (out, out_act) if gelu else out
+
+
+def estmm(dy, x, route, dy_per_slot, x_per_slot, out=None, out_dtype=torch.float32, accumulate=False):
+    """dw[e][o][i] (+)= sum over routed (slot, token) of dy[.., o] * x[.., i]  -> [E, out, in]."""
+    _dev(dy, x, out)
+    T, k, E = route.T, route.k, route.E
+    dy = dy.contiguous()
+    x = x.contiguous()
+    assert dy.dtype == x.dtype
+    out_dim, in_dim = dy.shape[-1], x.shape[-1]
+    assert tuple(dy.shape) == ((k, T, out_dim) if dy_per_slot else (T, out_dim))
+    assert tuple(x.shape) == ((k, T, in_dim) if x_per_slot else (T, in_dim))
+    if out is None:
+        assert not accumulate
+        out = torch.empty(E, out_dim, in_dim, dtype=out_dtype, device=x.device)
+    rc = _lib.load().hexa_estmm(_ptr(out), _ptr(dy), _ptr(x), _ptr(route.blob), int(bool(dy_per_slot)),
+                                int(bool(x_per_slot)), int(bool(accumulate)), T, k, out_dim, in_dim, E, _dt(x),
+                                _dt(out), _stream())
+    _lib.check(rc, "hexa_estmm")
+    return out
+
+
+def ess(dy, route, dy_per_slot, out=None, out_dtype=torch.float32, accumulate=False):
+    """db[e][o] (+)= sum over routed (slot, token) of dy[.., o] -> [E, out]."""
+    _dev(dy, out)
+    T, k, E = route.T, route.k, route.E
+    dy = dy.contiguous()
+    out_dim = dy.shape[-1]
+    assert tuple(dy.shape) == ((k, T, out_dim) if dy_per_slot else (T, out_dim))
+    if out is None:
+        assert not accumulate
+        out = torch.empty(E, out_dim, dtype=out_dtype, device=dy.device)
+    rc = _lib.load().hexa_ess(_ptr(out), _ptr(dy), _ptr(route.blob), int(bool(dy_per_slot)), int(bool(accumulate)),
+                              T, k, out_dim, E, _dt(dy), _dt(out), _stream())
+    _lib.check(rc, "hexa_ess")
+    return out
+
+
+def gelu_bwd(dy2, y1):
+    """dy1 = dy2 * gelu'(y1) (erf form)."""
+    _dev(dy2, y1)
+    dy2 = dy2.contiguous()
+    y1 = y1.contiguous()
+    assert dy2.shape == y1.shape and dy2.dtype == y1.dtype
+    out = torch.empty_like(dy2)
+    rc = _lib.load().hexa_gelu_bwd(_ptr(out), _ptr(dy2), _ptr(y1), dy2.numel(), _dt(dy2), _stream())
+    _lib.check(rc, "hexa_gelu_bwd")
+    return out

@@ -1,0 +1,121 @@
+"""The reference extension's five operators, same names and argument lists, on the HIP library.
+
+Mirrors the pybind module `hexa_moe_cuda` of the reference (hexa_moe_cuda/hexa_moe/torch/
+hexa_moe_ops.cpp:277-301): TOKEN_COUNT, TOKEN_ASSIGN, ESMM_TENSOR_CORE, FUSED_GRAD,
+FUSED_GRAD_NO_BIAS.  All results are written in place into caller-allocated tensors; the matmul
+results are accumulated (+=) as in the reference, whose callers zero them first
+(impls/layers.py:230-231, 404-405, 432-436).
+
+Differences that a caller can observe:
+  * segments are not padded: expanded_tokens_per_expert is the exact exclusive prefix, so the lists
+    the caller sizes from its last entry (impls/layers.py:238) have exactly num_tokens entries.
+    set_pad(16) switches TOKEN_COUNT / TOKEN_ASSIGN to the reference's 16-padded format; the matmul
+    ops accept unpadded lists only.
+  * the order inside a segment is ascending token id (the reference's depends on atomics).
+  * element types come from the tensors; the *_dtype_full flags are checked against them.  bf16 is
+    accepted wherever fp16 is.
+  * unsupported combinations raise instead of printing and returning.
+"""
+import torch
+
+from hexa_moe import _lib, ops
+
+_pad = 1
+
+
+def set_pad(pad):
+    """Segment granularity of TOKEN_COUNT / TOKEN_ASSIGN (1 = unpadded, 16 = the reference's)."""
+    global _pad
+    if int(pad) < 1:
+        raise ValueError("pad must be >= 1")
+    _pad = int(pad)
+
+
+def _scratch(num_tokens, num_routings, device):
+    units = max(1, -(-int(num_tokens) // _lib.HEXA_ROUTE_UNIT))
+    return torch.empty(units * int(num_routings), dtype=torch.int32, device=device)
+
+
+def _i32(t, what):
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise TypeError(f"{what} must be a contiguous int32 tensor")
+    ops._dev(t)
+    return t
+
+
+def TOKEN_COUNT(tokens_per_expert, expanded_tokens_per_expert, routings, num_tokens, num_routings):
+    _i32(tokens_per_expert, "tokens_per_expert"); _i32(expanded_tokens_per_expert, "expanded_tokens_per_expert")
+    _i32(routings, "routings")
+    assert tokens_per_expert.numel() >= num_routings and expanded_tokens_per_expert.numel() >= num_routings + 1
+    assert routings.numel() >= num_tokens
+    scratch = _scratch(num_tokens, num_routings, routings.device)
+    rc = _lib.load().hexa_token_count(tokens_per_expert.data_ptr(), expanded_tokens_per_expert.data_ptr(),
+                                      routings.data_ptr(), int(num_tokens), int(num_routings), _pad,
+                                      scratch.data_ptr(), ops._stream())
+    _lib.check(rc, "TOKEN_COUNT")
+
+
+def TOKEN_ASSIGN(token_idx_list, expert_idx_list, expanded_tokens_per_expert, routings, num_tokens, num_routings):
+    _i32(token_idx_list, "token_idx_list"); _i32(expert_idx_list, "expert_idx_list")
+    _i32(expanded_tokens_per_expert, "expanded_tokens_per_expert"); _i32(routings, "routings")
+    scratch = _scratch(num_tokens, num_routings, routings.device)
+    rc = _lib.load().hexa_token_assign(token_idx_list.data_ptr(), expert_idx_list.data_ptr(),
+                                       expanded_tokens_per_expert.data_ptr(), routings.data_ptr(), int(num_tokens),
+                                       int(num_routings), scratch.data_ptr(), ops._stream())
+    _lib.check(rc, "TOKEN_ASSIGN")
+
+
+def _route(token_idx_list, expert_idx_list, num_tokens, top_k, num_routings):
+    _i32(token_idx_list, "token_idx_list"); _i32(expert_idx_list, "expert_idx_list")
+    if token_idx_list.numel() != num_tokens * top_k or expert_idx_list.numel() != num_tokens * top_k:
+        raise NotImplementedError(
+            "the matmul operators take unpadded lists (top_k * num_tokens entries); build them with pad 1")
+    return ops.route_from_lists(token_idx_list, expert_idx_list, int(num_tokens), int(top_k), int(num_routings))
+
+
+def _check_flag(t, full, what):
+    if (t.dtype == torch.float32) != bool(full):
+        raise TypeError(f"{what}: dtype flag does not match the tensor ({t.dtype})")
+
+
+def ESMM_TENSOR_CORE(result, tokens, weights, bias, token_idx_list, expert_idx_list, num_expanded_tokens,
+                     x_dtype_full, w_dtype_full, b_dtype_full, m2s, num_tokens, top_k, num_in_dims, num_out_dims,
+                     num_routings):
+    T, k, E = int(num_tokens), int(top_k), int(num_routings)
+    _check_flag(tokens, x_dtype_full, "tokens"); _check_flag(weights, w_dtype_full, "weights")
+    route = _route(token_idx_list, expert_idx_list, T, k, E)
+    x = tokens.reshape((k, T, num_in_dims) if m2s else (T, num_in_dims))
+    w = weights.reshape(E, num_in_dims, num_out_dims)
+    b = bias.reshape(E, num_out_dims) if bias is not None and bias.numel() > 0 else None
+    out = result.reshape((T, num_out_dims) if m2s else (k, T, num_out_dims))
+    assert out.data_ptr() == result.data_ptr(), "result must be contiguous"
+    ops.esmm(x, w, b, route, bool(m2s), _lib.HEXA_W_IN_OUT, out=out, accumulate=True)
+
+
+def _fused(j_b, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, m2s, num_tokens, top_k, num_in_dims,
+           num_out_dims, num_routings):
+    T, k, E = int(num_tokens), int(top_k), int(num_routings)
+    route = _route(token_idx_list, expert_idx_list, T, k, E)
+    for t in (j_x, j_w, j_y, w, x) + ((j_b,) if j_b is not None else ()):
+        ops._dev(t)
+        if not t.is_contiguous():
+            raise TypeError("FUSED_GRAD: tensors must be contiguous")
+    rc = _lib.load().hexa_fused_grad(
+        j_b.data_ptr() if j_b is not None else None, j_x.data_ptr(), j_w.data_ptr(), j_y.data_ptr(), w.data_ptr(),
+        x.data_ptr(), route.blob.data_ptr(), int(bool(m2s)), 1, T, k, int(num_in_dims), int(num_out_dims), E,
+        ops._dt(j_y), ops._dt(w), ops._dt(j_x), ops._dt(j_w), ops._dt(j_b) if j_b is not None else 0, ops._stream())
+    _lib.check(rc, "FUSED_GRAD")
+
+
+def FUSED_GRAD(j_b, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, num_expanded_tokens, x_dtype_full,
+               w_dtype_full, m2s, num_tokens, top_k, num_in_dims, num_out_dims, num_routings):
+    _check_flag(j_y, x_dtype_full, "j_y"); _check_flag(w, w_dtype_full, "w")
+    _fused(j_b, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, m2s, num_tokens, top_k, num_in_dims,
+           num_out_dims, num_routings)
+
+
+def FUSED_GRAD_NO_BIAS(j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, num_expanded_tokens, x_dtype_full,
+                       w_dtype_full, m2s, num_tokens, top_k, num_in_dims, num_out_dims, num_routings):
+    _check_flag(j_y, x_dtype_full, "j_y"); _check_flag(w, w_dtype_full, "w")
+    _fused(None, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, m2s, num_tokens, top_k, num_in_dims,
+           num_out_dims, num_routings)

@@ -1,0 +1,155 @@
+/* libhexa_moe_hip.so -- C ABI of the MI355X (gfx950) expert-specific operators.
+ *
+ * Plain pointers and sizes only; every pointer except the layout struct is a DEVICE pointer owned
+ * by the caller; nothing here allocates, frees, synchronises with the host or reads device memory
+ * back.  Every entry point enqueues its kernels on `stream` (a hipStream_t passed as void*; NULL is
+ * the null stream) and returns immediately with 0 (HEXA_OK) or a negative HEXA_ERR_* code;
+ * hexa_last_error() then holds a message (thread-local).  The library never exits the process.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the HEXA-MoE
+ * repository, hexa_moe_cuda/hexa_moe/...).
+ */
+#ifndef HEXA_MOE_HIP_H
+#define HEXA_MOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HEXA_ABI_VERSION 1
+
+/* element types */
+#define HEXA_F32 0
+#define HEXA_F16 1
+#define HEXA_BF16 2
+
+/* expert weight layouts accepted by hexa_esmm */
+#define HEXA_W_IN_OUT 0 /* w[E][in][out]  (what the reference's ESMM_TENSOR_CORE takes)            */
+#define HEXA_W_OUT_IN 1 /* w[E][out][in]  (nn.Linear style; what FUSED_GRAD takes for its `w`)      */
+
+/* epilogue activations of hexa_esmm */
+#define HEXA_ACT_NONE 0
+#define HEXA_ACT_GELU 1 /* out_act = gelu_erf(out), written next to the pre-activation `out`        */
+
+/* return codes */
+#define HEXA_OK 0
+#define HEXA_ERR_ARG (-1)         /* null pointer, negative size, inconsistent flags                */
+#define HEXA_ERR_UNSUPPORTED (-2) /* dtype combination or dimension granularity not implemented     */
+#define HEXA_ERR_LAUNCH (-3)      /* the HIP runtime refused a launch                               */
+
+/* Rows per row-tile of the gathered-row kernels; the routing pass emits one tile record per
+ * HEXA_TILE_ROWS rows of every (slot, expert) segment. */
+#define HEXA_TILE_ROWS 128
+/* Tokens handled by one wavefront in the routing pass. */
+#define HEXA_ROUTE_UNIT 512
+
+/* ------------------------------------------------------------------------------------------------
+ * Routing metadata ("route blob"): ONE caller-owned int32 device buffer per MoE depth that every
+ * operator below consumes.  hexa_route_layout_get() gives the size and the position (in int32
+ * units) of each part so the host can slice it:
+ *   counts     [k][E]        tokens per expert per routing slot
+ *   offsets    [k][E+1]      exclusive prefix of counts (unpadded; offsets[s][E] == T)
+ *   token_ids  [k][T]        token ids grouped by expert, ascending inside a segment (stable)
+ *   expert_ids [k][T]        expert of each list position (the reference's expert_idx_list)
+ *   tile_count [k]           number of row tiles of the slot
+ *   tile_info  [k][mt_ub][4] {expert, first list position, rows (<=HEXA_TILE_ROWS), 0}
+ *   scratch    [k][units][E] per-wavefront histograms of the routing pass
+ * The buffer may be shared by all MoE depths of a model (sized for the largest T*k): its contents
+ * are rebuilt by hexa_route_build for each depth and reused by that depth's forward and backward
+ * operators.
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct hexa_route_layout {
+    int64_t counts, offsets, token_ids, expert_ids, tile_count, tile_info, scratch;
+    int64_t total_ints; /* size of the blob in int32 elements */
+    int32_t mt_ub;      /* row-tile upper bound per slot: T/HEXA_TILE_ROWS + E                      */
+    int32_t units;      /* wavefront units per slot: ceil(T/HEXA_ROUTE_UNIT)                        */
+} hexa_route_layout;
+
+int hexa_route_layout_get(int num_tokens, int top_k, int num_experts, hexa_route_layout* out);
+
+/* Routing segment pass: histogram + exclusive scan + stable scatter, all slots in one call, no
+ * padding, no host round trip.  Element (t, s) of the routing choice is read at
+ * routing[t*token_stride + s*slot_stride]; `routing_is_i64` selects int64 (torch.topk's output) or
+ * int32 elements.  Ids outside [0, E) are skipped.
+ * Replaces TOKEN_COUNT + TOKEN_ASSIGN: torch/hexa_moe_ops.cpp:9-43 -> launch_count / launch_assign,
+ * kernels/shared_cuda_core.cu:126-182, 284-333, and the per-slot Python loop impls/layers.py:233-251. */
+int hexa_route_build(const void* routing, int routing_is_i64, int64_t token_stride, int64_t slot_stride,
+                     int num_tokens, int top_k, int num_experts, int32_t* route, void* stream);
+
+/* The two reference ops one to one (a single routing slot, contiguous int32 routing[T]).
+ * `pad` is the segment granularity: 16 reproduces the reference's expanded_tokens_per_expert
+ * (shared_cuda_core.cu:165-171), 1 gives the exact prefix.  `scratch` holds
+ * ceil(T/HEXA_ROUTE_UNIT)*E int32.  token/expert lists: only real positions are written; padding
+ * positions keep what the caller filled in (-1 in the reference, impls/layers.py:238-239).
+ * Replaces launch_count (include/hexa_moe.h:3-10) and launch_assign (include/hexa_moe.h:12-20). */
+int hexa_token_count(int32_t* tokens_per_expert, int32_t* expanded_tokens_per_expert, const int32_t* routing,
+                     int num_tokens, int num_experts, int pad, int32_t* scratch, void* stream);
+int hexa_token_assign(int32_t* token_idx_list, int32_t* expert_idx_list,
+                      const int32_t* expanded_tokens_per_expert, const int32_t* routing, int num_tokens,
+                      int num_experts, int32_t* scratch, void* stream);
+
+/* Build a route blob from reference-style lists (k slots of exactly T entries each, grouped by
+ * expert, no padding): what a caller holding token_idx_list / expert_idx_list from the two ops above
+ * (pad = 1) passes on to the operators.  Replaces the host-side rebuild of expert_start_list in
+ * launch_fused_grad_* (kernels/fused_ops_full.cu:486-512). */
+int hexa_route_from_lists(const int32_t* token_idx_list, const int32_t* expert_idx_list, int num_tokens,
+                          int top_k, int num_experts, int32_t* route, void* stream);
+
+/* ESMM: out[(s),t,:] (+)= x[(s),t,:] . W[e_s(t)] + bias[e_s(t)] over all routed (slot, token) pairs.
+ *   m2s == 0: x [T,in] shared by the slots, out [k,T,out]      (fc1 of the MoE FFN)
+ *   m2s != 0: x [k,T,in] per slot,          out [T,out] = sum over slots (fc2; deterministic order)
+ * w_layout selects w[E][in][out] or w[E][out][in]; bias [E][out] may be NULL.  x_dt is F32 (then w,
+ * bias and out must be F32: true-fp32 MFMA path) or F16/BF16 (w may be the same 16-bit type or F32,
+ * fp32 accumulation; out may be that 16-bit type or F32).  accumulate != 0 adds into `out`.
+ * act == HEXA_ACT_GELU additionally writes gelu(out) to out_act (same shape/dtype as out; m2s == 0).
+ * Dimension granularity: in and out multiples of 8 (16-bit) / 4 (fp32).
+ * Replaces ESMM_TENSOR_CORE (torch/hexa_moe_ops.cpp:45-117) -> launch_esmm_accum_shared_tensor_{full,
+ * mix,half} (include/hexa_moe.h:22-72, kernels/esmm_full.cu:249-300), and with w_layout OUT_IN the
+ * ESMM task of FUSED_GRAD (kernels/fused_ops_full.cu:117-247). */
+int hexa_esmm(void* out, const void* x, const void* w, const void* bias, const int32_t* route, int m2s,
+              int w_layout, int accumulate, int num_tokens, int top_k, int in_dim, int out_dim,
+              int num_experts, int x_dt, int w_dt, int bias_dt, int out_dt, int act, void* out_act,
+              void* stream);
+
+/* ESTMM: dw[e][o][i] (+)= sum over slots s and tokens t routed to e of dy[(s),t,o] * x[(s),t,i].
+ * dy_per_slot / x_per_slot say whether the operand is [k,T,*] (1) or [T,*] shared by the slots (0).
+ * dt is the element type of dy and x (F32, F16 or BF16); dw_dt is F32 or dt.  Experts without tokens
+ * get exact zeros (or are left untouched when accumulating).
+ * Replaces the ESTMM task of FUSED_GRAD (kernels/fused_ops_full.cu:248-371). */
+int hexa_estmm(void* dw, const void* dy, const void* x, const int32_t* route, int dy_per_slot, int x_per_slot,
+               int accumulate, int num_tokens, int top_k, int out_dim, int in_dim, int num_experts, int dt,
+               int dw_dt, void* stream);
+
+/* ESS: db[e][o] (+)= sum over slots and tokens routed to e of dy[(s),t,o].
+ * Replaces the ESS task of FUSED_GRAD (kernels/fused_ops_full.cu:372-431). */
+int hexa_ess(void* db, const void* dy, const int32_t* route, int dy_per_slot, int accumulate, int num_tokens,
+             int top_k, int out_dim, int num_experts, int dt, int db_dt, void* stream);
+
+/* The reference's fused backward of one expert linear:
+ *   j_x[(s),t,:in] (+)= j_y[(s),t,:out] . w[e]      w [E][out][in]
+ *   j_w[e]         (+)= sum j_y^T x                 j_w [E][out][in]
+ *   j_b[e]         (+)= sum j_y                     j_b [E][out], NULL = FUSED_GRAD_NO_BIAS
+ *   m2s == 0: j_y [T,out] shared, x and j_x [k,T,in]     (fc2 call, impls/layers.py:409-416)
+ *   m2s != 0: j_y [k,T,out], x [T,in] shared, j_x [T,in] (fc1 call, impls/layers.py:435-451)
+ * act_dt: element type of j_y and x; w_dt: of w; jx_dt / jw_dt / jb_dt: of the results.
+ * Replaces FUSED_GRAD / FUSED_GRAD_NO_BIAS (torch/hexa_moe_ops.cpp:119-275) ->
+ * launch_fused_grad_{bias,no_bias}_{full,mix,half} (include/hexa_moe.h:74-181). */
+int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y, const void* w, const void* x,
+                    const int32_t* route, int m2s, int accumulate, int num_tokens, int top_k, int in_dim,
+                    int out_dim, int num_experts, int act_dt, int w_dt, int jx_dt, int jw_dt, int jb_dt,
+                    void* stream);
+
+/* Elementwise backward of the fused GELU: dy1 = dy2 * gelu'(y1), n elements of type dt.  The
+ * reference evaluates act' with torch.autograd.functional.jacobian (impls/layers.py:281-283,427). */
+int hexa_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, void* stream);
+
+const char* hexa_last_error(void);
+int hexa_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HEXA_MOE_HIP_H */

@@ -1,0 +1,107 @@
+"""Routing segment pass on the GPU vs the CPU oracle: bit-exact counts, offsets and token lists."""
+import numpy as np
+import pytest
+import torch
+
+from _util import make_routing
+from oracle import hexa_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # T, E, k, skew, empty
+    (1, 1, 1, None, 0),
+    (7, 3, 1, None, 0),
+    (64, 8, 2, None, 0),
+    (513, 5, 3, None, 0),
+    (2048, 8, 1, None, 0),
+    (4608, 32, 1, None, 0),
+    (18432, 32, 2, None, 0),
+    (4099, 64, 2, "zipf", 6),
+    (32768, 64, 2, "zipf", 4),
+    (1000, 16, 2, "one", 0),
+    (3000, 300, 2, None, 0),
+]
+
+
+@pytest.mark.parametrize("T,E,k,skew,empty", CASES)
+@pytest.mark.parametrize("as_i64", [False, True])
+def test_route_build_matches_oracle(dev, T, E, k, skew, empty, as_i64):
+    from hexa_moe import ops
+    print(f"case T={T} E={E} k={k} skew={skew} i64={as_i64}", flush=True)
+    routing = make_routing(T, E, k, seed=100 + T + E, skew=skew, empty=empty)
+    counts, offsets, token_ids = O.route_build(routing, E)
+    r = routing if as_i64 else routing.to(torch.int32)
+    route = ops.route_build(r.to(dev), E)
+    torch.cuda.synchronize()
+    assert torch.equal(route.counts.cpu(), counts)
+    assert torch.equal(route.offsets.cpu(), offsets)
+    assert torch.equal(route.token_ids.cpu(), token_ids)
+    # expert of every list position, and the row-tile records the matmul kernels walk
+    exp = route.expert_ids.cpu()
+    tiles = route.tile_info.cpu()
+    ntile = route.tile_count.cpu()
+    for s in range(k):
+        assert torch.equal(exp[s], routing[token_ids[s].long(), s].to(torch.int32))
+        want = []
+        for e in range(E):
+            c, o = int(counts[s, e]), int(offsets[s, e])
+            for j in range(0, c, 128):
+                want.append((e, o + j, min(128, c - j), 0))
+        assert int(ntile[s]) == len(want)
+        got = [tuple(int(v) for v in row) for row in tiles[s, :len(want)]]
+        assert got == want
+    if skew == "zipf":
+        assert int((counts.sum(0) == 0).sum()) >= empty
+
+
+def test_route_transposed_slots_and_noncontiguous(dev):
+    """k contiguous slot vectors ([k,T] storage) give the same lists as [T,k] storage."""
+    from hexa_moe import ops
+    routing = make_routing(3000, 16, 2, seed=5)
+    a = ops.route_build(routing.to(dev), 16)
+    b = ops.route_build(routing.t().contiguous().to(dev).t(), 16)
+    torch.cuda.synchronize()
+    assert torch.equal(a.token_ids, b.token_ids) and torch.equal(a.offsets, b.offsets)
+
+
+def test_route_out_of_range_ids_are_skipped(dev):
+    from hexa_moe import ops
+    routing = make_routing(1000, 8, 1, seed=6).to(torch.int32)
+    routing[::7, 0] = 8
+    routing[3::11, 0] = -1
+    keep = ((routing[:, 0] >= 0) & (routing[:, 0] < 8)).nonzero().flatten()
+    route = ops.route_build(routing.to(dev), 8)
+    torch.cuda.synchronize()
+    n = int(route.offsets[0, 8])
+    assert n == keep.numel()
+    want = keep[torch.sort(routing[keep, 0], stable=True).indices].to(torch.int32)
+    assert torch.equal(route.token_ids[0, :n].cpu(), want)
+
+
+@pytest.mark.parametrize("pad", [1, 16])
+def test_legacy_count_assign(dev, pad):
+    """TOKEN_COUNT / TOKEN_ASSIGN one to one, including the reference's 16-padded format."""
+    import hexa_moe_cuda
+    from oracle import route_oracle as RO
+    T, E = 5000, 32
+    routing = make_routing(T, E, 1, seed=9, skew="zipf", empty=3)[:, 0].to(torch.int32)
+    c_ref, x_ref = RO.token_count(routing.numpy(), E, pad)
+    t_ref, e_ref = RO.token_assign(routing.numpy(), E, x_ref)
+    r = routing.to(dev)
+    cnt = torch.zeros(E, dtype=torch.int32, device=dev)
+    expd = torch.zeros(E + 1, dtype=torch.int32, device=dev)
+    hexa_moe_cuda.set_pad(pad)
+    try:
+        hexa_moe_cuda.TOKEN_COUNT(cnt, expd, r, T, E)
+        P = int(expd[-1].item())
+        tok = torch.zeros(P, dtype=torch.int32, device=dev) - 1
+        exp = torch.zeros(P, dtype=torch.int32, device=dev) - 1
+        hexa_moe_cuda.TOKEN_ASSIGN(tok, exp, expd, r, T, E)
+    finally:
+        hexa_moe_cuda.set_pad(1)
+    torch.cuda.synchronize()
+    assert np.array_equal(cnt.cpu().numpy(), c_ref)
+    assert np.array_equal(expd.cpu().numpy(), x_ref)
+    assert np.array_equal(tok.cpu().numpy(), t_ref)
+    assert np.array_equal(exp.cpu().numpy(), e_ref)

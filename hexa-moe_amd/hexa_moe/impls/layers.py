@@ -1,0 +1,167 @@
+"""Autograd functions of the cascaded MoE (reference: hexa_moe_cuda/hexa_moe/impls/layers.py).
+
+FusedMoE_Shared_CudaCore is the MoE FFN of one depth in data-centric mode on one GPU: the ten steps
+of the paper's formula table, each an expert-specific operator of libhexa_moe_hip.so:
+
+    forward   1  y1 = ESMM(x, W1, b1)            3  y = ESMM(act(y1), W2, b2), summed over the slots
+    backward  4  db2 = ESS(dy)                    5  dW2 = ESTMM(act(y1), dy)     6  dy2 = ESMM(dy, W2^T)
+              7  dy1 = dy2 * act'(y1)             8  db1 = ESS(dy1)               9  dW1 = ESTMM(dy1, x)
+              10 dx = ESMM(dy1, W1^T), summed over the slots
+
+Against the reference (layers.py:99-277, 280-474) on the same math:
+  * weights are read in their parameter layout ([E,h,d_in], [E,h,d_out]); nothing is concatenated,
+    permuted or copied per call (layers.py:119-122, 307-309, 412, 438 copy every expert weight);
+  * results are written in their final type; no fp32 staging buffers, zero-fills or cast kernels
+    (layers.py:230-231, 260, 275);
+  * the routing lists are built once per depth on the device, without .item() (layers.py:238), and the
+    same metadata serves all six matmuls, both ESS calls and the backward;
+  * gradients are returned for the Parameters that were passed in (the reference passes `.data`, so
+    its expert gradients are dropped: cascaded_moe.py:553-559);
+  * the activation is evaluated once: the backward differentiates the forward's own graph (or the
+    fused GELU), not a second evaluation (layers.py:281-283, 407), so stochastic activations
+    (dropout) use one mask.
+"""
+from typing import Any
+
+import torch
+import torch.nn.functional as F
+
+from .. import _lib, ops
+from . import losses
+
+
+def is_plain_gelu(fn) -> bool:
+    """True for activations known to be the exact (erf) GELU, which the kernels fuse."""
+    return fn is F.gelu or getattr(fn, "hexa_fused", None) == "gelu"
+
+
+def fused_gelu(x):
+    """Marker activation: pass `activation_fn=fused_gelu` to get the fused GELU epilogue."""
+    return F.gelu(x)
+
+
+fused_gelu.hexa_fused = "gelu"
+
+
+class MLP_Implement:
+    """Dense FFN depth (reference: layers.py:25-95): y = act(x fc1_w^T + b1) fc2_w + b2 with
+    fc1_w [h, d_in], fc2_w [h, d_out].  Plain differentiable PyTorch (rocBLAS GEMMs); on one GPU the
+    reference's gradient all-reduces are the identity."""
+
+    @staticmethod
+    def apply(config: Any, tokens_input, fc1_w, fc2_w, fc1_bias, fc2_bias):
+        dt = tokens_input.dtype
+        hid = F.linear(tokens_input, fc1_w.to(dt), fc1_bias.to(dt) if fc1_bias is not None else None)
+        out = config.activation_fn(hid) @ fc2_w.to(dt)
+        if fc2_bias is not None:
+            out = out + fc2_bias.to(dt)
+        return out
+
+
+def _weight_for(x, w):
+    """Kernels take weights in the tokens' 16-bit type or in fp32; anything else is converted."""
+    if w.dtype == x.dtype or (w.dtype == torch.float32 and x.dtype != torch.float32):
+        return w
+    return w.to(x.dtype)
+
+
+class FusedMoE_Shared_CudaCore(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx: Any, config: Any, tokens_input, fc1_w, fc2_w, fc1_bias, fc2_bias):
+        x = tokens_input.contiguous()
+        if not x.is_cuda:
+            raise RuntimeError("hexa_moe: the MoE FFN runs on the GPU only (no CPU fallback); move the module "
+                               "and its input to a HIP device")
+        E = int(config.num_global_experts)
+        T, d_in = x.shape
+        assert fc1_w.shape[0] == E and fc2_w.shape[0] == E and fc1_w.shape[2] == d_in
+        assert fc1_w.shape[1] == fc2_w.shape[1]
+
+        indices = config.indices_
+        routing = indices if torch.is_tensor(indices) else torch.stack([i.reshape(-1) for i in indices], dim=1)
+        blob = config.route_pool.slot(config.stage, T, routing.shape[1], E, x.device)
+        route = ops.route_build(routing, E, blob=blob)
+        if any(ctx.needs_input_grad):
+            config.route_pool.bind(config.stage, route)  # keep the slot until this call's backward is done
+
+        w1, w2 = _weight_for(x, fc1_w), _weight_for(x, fc2_w)
+        act = config.activation_fn
+        fused = is_plain_gelu(act)
+        ctx.act_graph = None
+        if fused:
+            y1, y2 = ops.esmm(x, w1, fc1_bias, route, False, _lib.HEXA_W_OUT_IN, gelu=True)
+        else:
+            y1 = ops.esmm(x, w1, fc1_bias, route, False, _lib.HEXA_W_OUT_IN)
+            if any(ctx.needs_input_grad):
+                with torch.enable_grad():
+                    y1_leaf = y1.detach().requires_grad_(True)
+                    y2_graph = act(y1_leaf)
+                ctx.act_graph = (y1_leaf, y2_graph)
+                y2 = y2_graph.detach()
+            else:
+                y2 = act(y1)
+            if y2.dtype != x.dtype:
+                y2 = y2.to(x.dtype)
+        y = ops.esmm(y2.contiguous(), w2, fc2_bias, route, True, _lib.HEXA_W_IN_OUT)
+
+        ctx.config = config
+        ctx.route = route
+        ctx.fused = fused
+        ctx.has_b1, ctx.has_b2 = fc1_bias is not None, fc2_bias is not None
+        ctx.param_dtypes = (fc1_w.dtype, fc2_w.dtype,
+                            fc1_bias.dtype if fc1_bias is not None else None,
+                            fc2_bias.dtype if fc2_bias is not None else None)
+        ctx.save_for_backward(x, y1, y2 if fused else None, w1, w2)
+        return y
+
+    @staticmethod
+    def backward(ctx: Any, j_tokens_output):
+        x, y1, y2, w1, w2 = ctx.saved_tensors
+        route = ctx.route
+        dy = j_tokens_output.contiguous().to(x.dtype)
+        need_x, need_w1, need_w2, need_b1, need_b2 = ctx.needs_input_grad[1:6]
+        dt_w1, dt_w2, dt_b1, dt_b2 = ctx.param_dtypes
+        if not ctx.fused:
+            y1_leaf, y2_graph = ctx.act_graph
+            y2 = y2_graph.detach().to(x.dtype).contiguous()
+
+        def grad_dtype(param_dtype):  # fp32 master weights get fp32 grads, 16-bit weights 16-bit grads
+            return torch.float32 if param_dtype == torch.float32 else x.dtype
+
+        db2 = dw2 = db1 = dw1 = dx = None
+        if ctx.has_b2 and need_b2:
+            db2 = ops.ess(dy, route, False, out_dtype=grad_dtype(dt_b2)).to(dt_b2)
+        if need_w2:
+            # [E, h, d_out]: the per-slot operand act(y1) supplies the rows of dW2
+            dw2 = ops.estmm(y2, dy, route, True, False, out_dtype=grad_dtype(dt_w2)).to(dt_w2)
+        if need_x or need_w1 or (ctx.has_b1 and need_b1):
+            dy2 = ops.esmm(dy, w2, None, route, False, _lib.HEXA_W_OUT_IN)
+            if ctx.fused:
+                dy1 = ops.gelu_bwd(dy2, y1)
+            else:
+                (dy1,) = torch.autograd.grad(y2_graph, y1_leaf, dy2.to(y2_graph.dtype))
+                dy1 = dy1.to(x.dtype).contiguous()
+            if ctx.has_b1 and need_b1:
+                db1 = ops.ess(dy1, route, True, out_dtype=grad_dtype(dt_b1)).to(dt_b1)
+            if need_w1:
+                dw1 = ops.estmm(dy1, x, route, True, False, out_dtype=grad_dtype(dt_w1)).to(dt_w1)
+            if need_x:
+                dx = ops.esmm(dy1, w1, None, route, True, _lib.HEXA_W_IN_OUT)
+        ctx.act_graph = None
+        ctx.config.stage = ctx.config.stage - 1
+        return (None, dx, dw1, dw2, db1, db2)
+
+
+def topk_and_loss(scores, top_k, loss_fn=losses.gshard_loss):
+    """Top-k expert choice as one [T,k] int64 tensor (what the routing pass reads directly) and the
+    auxiliary loss."""
+    top_k = min(int(top_k), int(scores.size(1)))
+    topk_indices = torch.topk(scores, top_k, dim=1).indices
+    l_loss = loss_fn(scores, topk_indices) if loss_fn is not None else None
+    return topk_indices, l_loss
+
+
+def simplified_extract_critical(scores, top_k, loss_fn=losses.gshard_loss):
+    """Same contract as the reference's helper (layers.py:476-484): the k index vectors and the loss."""
+    topk_indices, l_loss = topk_and_loss(scores, top_k, loss_fn)
+    return [col.reshape(-1) for col in topk_indices.unbind(dim=1)], l_loss

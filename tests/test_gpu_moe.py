@@ -1,0 +1,193 @@
+"""MoE_Cascaded on the GPU vs the CPU oracle: forward, input gradient and every parameter gradient.
+
+The module runs the HIP operators through the C ABI; the oracle evaluates the formula table on the
+CPU in fp32/fp64 from the same parameters and the module's own routing decision (the top-k indices
+are produced by the same torch ops on both sides, so they are compared bit-exactly)."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from _util import TOL, assert_close
+from oracle import hexa_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _module(dims, moe_idx, E, k, bias=True, act=None, dtype=torch.float32, seed=1234, noise=1.0):
+    from hexa_moe import moe as hmoe
+    torch.manual_seed(seed)
+    m = hmoe.MoE_Cascaded(gate_type={'type': 'top', 'k': k, 'gate_noise': noise, 'fp32_gate': True},
+                          model_dim_list=dims, moe_idx_list=moe_idx, mlp_ratio=4, num_global_experts=E,
+                          total_depth=len(dims), data_centric=True, mlp_fc1_bias=bias, mlp_fc2_bias=bias,
+                          activation_fn=act if act is not None else (lambda x: F.gelu(x)))
+    g = torch.Generator().manual_seed(seed)
+    for name, p in m.named_parameters():          # U(+-1/sqrt(fan_in)) from the seed
+        fan_in = p.shape[-1] if name.startswith(("batched_fc1_w", "mlp_fc1_w", "gates")) else p.shape[-2] if p.dim() > 1 else p.shape[-1]
+        p.data.copy_((torch.rand(p.shape, generator=g) * 2 - 1) / fan_in ** 0.5)
+    return m
+
+
+def _oracle_depth(m, i, x, routing, dy, act, rd):
+    W1, W2 = m.batched_fc1_w[i].detach().cpu().to(rd), m.batched_fc2_w[i].detach().cpu().to(rd)
+    b1 = m.batched_fc1_bias[i].detach().cpu().to(rd) if m.has_fc1_bias else None
+    b2 = m.batched_fc2_bias[i].detach().cpu().to(rd) if m.has_fc2_bias else None
+    y, y1, _ = O.moe_ffn_forward(x.to(rd), W1, W2, b1, b2, routing, act)
+    grads = O.moe_ffn_backward(dy.to(rd), x.to(rd), y1, W1, W2, b1 is not None, b2 is not None, routing, act)
+    return y, grads
+
+
+def test_readme_config_fp32(dev):
+    """Tiny MoE_Cascaded as in the reference's README: dims 128 x4, MoE at depths 2 and 3, 8 experts,
+    top-1, gate noise 1.0, fp32, 2048 tokens, loss = sum(y) + l_aux, train mode."""
+    m = _module([128] * 4, [2, 3], E=8, k=1).to(dev).train()
+    g = torch.Generator().manual_seed(1234)
+    x0 = torch.randn(2048, 128, generator=g)
+    x = x0.to(dev).requires_grad_(True)
+    h = x
+    captured = []
+    aux = 0
+    for depth in range(4):
+        h_in = h
+        h, l_aux = m(depth, h)
+        if depth in (2, 3):
+            captured.append((depth, h_in, m.dispatch_params.indices_.clone(), h))
+            h.retain_grad(); h_in.retain_grad()
+            aux = aux + l_aux
+    (h.sum() + aux).backward()
+    torch.cuda.synchronize()
+    for depth, h_in, routing, h_out in captured:
+        i = m.moe_idx_list.index(depth)
+        r = routing.cpu()
+        # counts the device built are the bincount of the routing decision, bit for bit
+        y_ref, (dx, dW1, dW2, db1, db2) = _oracle_depth(m, i, h_in.detach().cpu(), r, h_out.grad.cpu(), F.gelu, torch.float64)
+        assert_close(h_out.detach(), y_ref, 1e-5, f"y depth {depth}")
+        assert_close(m.batched_fc1_w[i].grad, dW1, 1e-5, "dW1")
+        assert_close(m.batched_fc2_w[i].grad, dW2, 1e-5, "dW2")
+        assert_close(m.batched_fc1_bias[i].grad, db1, 1e-5, "db1")
+        assert_close(m.batched_fc2_bias[i].grad, db2, 1e-5, "db2")
+        if depth == 3:   # h_in.grad of depth 3 is purely the layer's dx (+ the gate's aux-loss path)
+            gate_free = h_in.grad.detach().cpu().double() - dx
+            assert gate_free.abs().max() < 1e-2   # what is left is the small l_aux gradient through the gate
+    assert x.grad is not None and m.gates[0].wg.weight.grad is not None
+    assert m.mlp_fc1_w[0].grad is not None
+
+
+@pytest.mark.parametrize("dtype,k,bias", [(torch.float32, 2, True), (torch.bfloat16, 1, True), (torch.bfloat16, 2, False),
+                                          (torch.float16, 2, True)])
+def test_single_depth_against_oracle(dev, dtype, k, bias):
+    E, d, T = 16, 256, 3000
+    m = _module([d], [0], E=E, k=k, bias=bias, noise=0.0).to(dev).to(dtype).eval()
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(T, d, generator=g).to(dtype)
+    dy = torch.randn(T, d, generator=g).to(dtype)
+    xd = x.to(dev).requires_grad_(True)
+    y, l_aux = m(0, xd)
+    routing = m.dispatch_params.indices_.cpu()
+    y.backward(dy.to(dev))
+    torch.cuda.synchronize()
+    assert y.dtype == dtype and l_aux.dim() == 0
+    # the device's per-expert counts equal the bincount of the decision
+    rd = torch.float64 if dtype == torch.float32 else torch.float32
+    y_ref, (dx, dW1, dW2, db1, db2) = _oracle_depth(m, 0, x, routing, dy, F.gelu, rd)
+    tol = TOL[dtype]
+    assert_close(y, y_ref, tol, "y")
+    assert_close(xd.grad, dx, tol, "dx")
+    assert_close(m.batched_fc1_w[0].grad, dW1, tol, "dW1")
+    assert_close(m.batched_fc2_w[0].grad, dW2, tol, "dW2")
+    if bias:
+        assert_close(m.batched_fc1_bias[0].grad, db1, tol, "db1")
+        assert_close(m.batched_fc2_bias[0].grad, db2, tol, "db2")
+    assert m.batched_fc1_w[0].grad.dtype == dtype
+
+
+def test_fused_gelu_equals_generic_activation_path(dev):
+    """F.gelu itself is recognised and fused; a lambda goes through autograd of the callable."""
+    E, d, T = 8, 128, 1500
+    a = _module([d], [0], E=E, k=2, act=F.gelu, noise=0.0).to(dev).eval()
+    b = _module([d], [0], E=E, k=2, act=lambda t: F.gelu(t), noise=0.0).to(dev).eval()
+    b.load_state_dict(a.state_dict())
+    x = torch.randn(T, d, device=dev)
+    outs = []
+    for m in (a, b):
+        xi = x.clone().requires_grad_(True)
+        y, _ = m(0, xi)
+        y.square().sum().backward()
+        outs.append((y.detach(), xi.grad, m.batched_fc1_w[0].grad, m.batched_fc2_bias[0].grad))
+    torch.cuda.synchronize()
+    for u, v in zip(*outs):
+        assert_close(u, v, 2e-5, "fused vs generic")
+
+
+def test_stochastic_activation_uses_one_mask(dev):
+    """dropout(gelu(x)) as in the Swin model: the backward must see the forward's mask, so the layer's
+    gradients equal those of the oracle evaluated with that same mask."""
+    E, d, T = 4, 128, 1024
+    masks = []
+
+    def act(t):
+        y = F.gelu(t)
+        mk = (torch.rand_like(y) > 0.3).to(y.dtype) / 0.7
+        masks.append(mk)
+        return y * mk
+
+    m = _module([d], [0], E=E, k=1, act=act, noise=0.0).to(dev).train()
+    x = torch.randn(T, d, device=dev, requires_grad=True)
+    y, _ = m(0, x)
+    dy = torch.randn_like(y)
+    y.backward(dy)
+    torch.cuda.synchronize()
+    assert len(masks) == 1, "the activation must be evaluated exactly once per forward+backward"
+    mk = masks[0].cpu().double()
+    routing = m.dispatch_params.indices_.cpu()
+    y_ref, (dx, dW1, dW2, db1, db2) = _oracle_depth(m, 0, x.detach().cpu(), routing, dy.cpu(), lambda t: F.gelu(t) * mk, torch.float64)
+    assert_close(y.detach(), y_ref, 1e-5, "y")
+    assert_close(x.grad, dx, 1e-5, "dx")
+    assert_close(m.batched_fc1_w[0].grad, dW1, 1e-5, "dW1")
+
+
+def test_autocast_bf16_with_fp32_master_weights(dev):
+    E, d, T = 8, 256, 2000
+    m = _module([d, d], [1], E=E, k=2, noise=0.0).to(dev).eval()
+    x = torch.randn(T, d, device=dev, requires_grad=True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        h, _ = m(0, x)
+        y, _ = m(1, h)
+    assert y.dtype == torch.float32 or y.dtype == x.dtype
+    dy = torch.randn_like(y)
+    h.retain_grad()
+    y.backward(dy)
+    torch.cuda.synchronize()
+    routing = m.dispatch_params.indices_.cpu()
+    hb = h.detach().to(torch.bfloat16).float().cpu()
+    W1 = m.batched_fc1_w[0].detach().to(torch.bfloat16).float().cpu()
+    W2 = m.batched_fc2_w[0].detach().to(torch.bfloat16).float().cpu()
+    b1, b2 = m.batched_fc1_bias[0].detach().cpu(), m.batched_fc2_bias[0].detach().cpu()
+    y_ref, y1, _ = O.moe_ffn_forward(hb, W1, W2, b1, b2, routing, F.gelu)
+    dx, dW1, dW2, db1, db2 = O.moe_ffn_backward(dy.to(torch.bfloat16).float().cpu(), hb, y1, W1, W2, True, True, routing, F.gelu)
+    assert_close(y.detach().float(), y_ref, 2e-2, "y")
+    assert m.batched_fc1_w[0].grad.dtype == torch.float32
+    assert_close(m.batched_fc1_w[0].grad, dW1, 2e-2, "dW1")
+    assert_close(m.batched_fc2_w[0].grad, dW2, 2e-2, "dW2")
+    assert_close(m.batched_fc2_bias[0].grad, db2, 2e-2, "db2")
+
+
+def test_route_pool_is_reused_across_steps_and_survives_pending_backward(dev):
+    E, d, T = 8, 128, 512
+    m = _module([d, d], [0, 1], E=E, k=1, noise=0.0).to(dev).eval()
+    pool = m.dispatch_params.route_pool
+    x = torch.randn(T, d, device=dev, requires_grad=True)
+    y, _ = m(0, x)
+    first = pool._slots[0][0]
+    y.sum().backward()
+    del y
+    y, _ = m(0, x)
+    assert pool._slots[0][0] is first, "a slot whose backward is done is reused, not reallocated"
+    y2, _ = m(0, x)   # the first call's backward is still pending: its metadata must not be overwritten
+    assert pool._slots[0][0] is not first
+    (y.sum() + y2.sum()).backward()
+    torch.cuda.synchronize()
+    with torch.no_grad():
+        m(1, x)
+        before = pool._slots[1][0]
+        m(1, x)
+        assert pool._slots[1][0] is before

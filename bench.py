@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X: a full MoE layer forward + backward at the Swin-MoE-S
+stage-3 shape (T=18432 tokens, d=384, h=1536, 32 experts, top-2, bf16 with fp32 accumulation).
+
+One step = gate projection + softmax + top-2 + auxiliary loss, the routing segment pass, fc1 ESMM with
+the fused GELU, fc2 ESMM, and the whole backward (2x ESS, 2x ESTMM, 2x backward ESMM, GELU') through the
+product's autograd function, with every input already resident in HBM.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import math
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "hexa-moe_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
+
+T, D, H, E, K_TOP = 18432, 384, 1536, 32, 2
+SEED = 1235
+
+
+def make_inputs(dev):
+    import torch
+    g = torch.Generator().manual_seed(SEED)
+    bf = torch.bfloat16
+    u = lambda shape, bound: (torch.rand(shape, generator=g) * 2 - 1) * bound  # noqa: E731
+    p = {
+        "x": torch.randn(T, D, generator=g).to(bf),
+        "W1": u((E, H, D), 1 / math.sqrt(D)).to(bf),      # [E,h,d_in]  (parameter layout)
+        "W2": u((E, H, D), 1 / math.sqrt(H)).to(bf),      # [E,h,d_out]
+        "b1": u((E, H), 1 / math.sqrt(D)).to(bf),
+        "b2": u((E, D), 1 / math.sqrt(H)).to(bf),
+        "wg": torch.randn(E, D, generator=g) / math.sqrt(D),          # fp32 gate: logits ~ N(0,1)
+        "ebias": 0.5 * torch.randn(E, generator=g),                   # per-expert bias -> uneven load
+        "dy": torch.randn(T, D, generator=g).to(bf),
+    }
+    return {k: v.to(dev) for k, v in p.items()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-events", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (data-centric mode, no expert or model sharding, no "
+                 "collectives); --gpus must be 1")
+
+    import torch
+    import torch.nn.functional as F
+    from types import SimpleNamespace
+
+    from hexa_moe import _lib, ops
+    from hexa_moe.impls import losses
+    from hexa_moe.impls.cascaded_moe import RoutePool
+    from hexa_moe.impls.layers import FusedMoE_Shared_CudaCore
+
+    _lib.load()  # no fallback: a missing library is an error
+    dev = torch.device("cuda:0")
+    p = make_inputs(dev)
+    leaves = ["x", "W1", "W2", "b1", "b2", "wg"]
+    for k in leaves:
+        p[k].requires_grad_(True)
+    cfg = SimpleNamespace(activation_fn=F.gelu, stage=0, num_global_experts=E, indices_=None, route_pool=RoutePool())
+    one = torch.ones((), device=dev)
+
+    def step():
+        for k in leaves:
+            p[k].grad = None
+        logits = F.linear(p["x"].float(), p["wg"]) + p["ebias"]
+        scores = F.softmax(logits, dim=1)
+        idx = torch.topk(scores, K_TOP, dim=1).indices
+        l_aux = losses.gshard_loss(scores, idx)
+        cfg.indices_, cfg.stage = idx, 0
+        y = FusedMoE_Shared_CudaCore.apply(cfg, p["x"], p["W1"], p["W2"], p["b1"], p["b2"])
+        torch.autograd.backward([y, l_aux], [p["dy"], one])
+        return y, idx
+
+    for _ in range(args.warmup):
+        step()
+    timer = None if args.no_kernel_events else ops.OpTimer()
+    ops.set_timer(timer)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        y, idx = step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ops.set_timer(None)
+    ms = (t1 - t0) * 1e3 / args.steps
+    flops_step = 12.0 * T * K_TOP * D * H
+    tokens_per_s = T / (ms * 1e-3)
+
+    # ---- per-kernel durations (events on the launch stream, taken inside the timed region) ----
+    kernels = {}
+    roofline = None
+    if timer is not None:
+        gemm = 2.0 * T * K_TOP * D * H
+        esz = 2  # bf16
+        alg = {  # algorithmic work per call: flop for the matmuls, bytes for the HBM-bound kernels
+            "route_build": ("hbm", T * K_TOP * 8 + T * K_TOP * 8 + K_TOP * (2 * E + 1) * 4),
+            "gelu_bwd": ("hbm", 3 * T * K_TOP * H * esz),
+            f"ess[{H},per_slot]": ("hbm", T * K_TOP * H * esz + E * H * esz),
+            f"ess[{D}]": ("hbm", T * K_TOP * D * esz + E * D * esz),
+        }
+        for label, vals in timer.durations().items():
+            avg_ms = statistics.mean(vals)
+            per_step = len(vals) / args.steps
+            kind, work = alg.get(label, ("mfma", gemm))
+            entry = {"avg_us": round(avg_ms * 1e3, 2), "calls_per_step": per_step, "bound": kind}
+            if kind == "mfma":
+                entry["tflops"] = round(work / (avg_ms * 1e-3) / 1e12, 1)
+                entry["frac"] = round(entry["tflops"] / PEAK_BF16_TFLOPS, 4)
+            else:
+                entry["gbs"] = round(work / (avg_ms * 1e-3) / 1e9, 1)
+                entry["frac"] = round(entry["gbs"] / PEAK_HBM_GBS, 4)
+            kernels[label] = entry
+        dom = max(kernels, key=lambda k: kernels[k]["avg_us"] * kernels[k]["calls_per_step"])
+        d = kernels[dom]
+        if d["bound"] == "mfma":
+            roofline = {"kernel": dom, "bound": "mfma", "achieved": d["tflops"], "peak": PEAK_BF16_TFLOPS,
+                        "unit": "TFLOP/s", "frac": d["frac"], "traffic": None}
+        else:
+            roofline = {"kernel": dom, "bound": "hbm", "achieved": d["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                        "frac": d["frac"], "traffic": None}
+
+    # ---- CPU baseline: the oracle's plain-PyTorch fp32 evaluation of the same layer on the host ----
+    cpu = None
+    parity = None
+    if not args.no_cpu_baseline:
+        from oracle import hexa_oracle as O
+        threads = min(16, os.cpu_count() or 1)
+        torch.set_num_threads(threads)
+        c = {k: p[k].detach().float().cpu() for k in ("x", "W1", "W2", "b1", "b2", "dy")}
+        routing = idx.cpu()
+        run = lambda: O.moe_layer_fwd_bwd_cpu(c["x"], c["W1"], c["W2"], c["b1"], c["b2"], routing, c["dy"], F.gelu)  # noqa: E731
+        run()
+        times = []
+        for _ in range(3):
+            a = time.perf_counter()
+            ref = run()
+            times.append(time.perf_counter() - a)
+        sec = statistics.median(times)
+        cpu = {"value": round(T / sec, 1), "unit": "tokens/s", "cores": threads, "kind": "port",
+               "gflops": round(flops_step / sec / 1e9, 1),
+               "sample": f"the full workload (T={T}, one layer fwd+bwd, fp32, per-expert index_select/mm/index_add), "
+                         f"1 warm-up + median of 3 on {threads} threads"}
+        names = ["y", "dx", "dW1", "dW2", "db1", "db2"]
+        got = [y, p["x"].grad, p["W1"].grad, p["W2"].grad, p["b1"].grad, p["b2"].grad]
+        # dx also carries the (tiny) auxiliary-loss gradient through the gate; it is left out of the check
+        parity = {n: float((g_.detach().float().cpu() - r).norm() / r.norm()) for n, g_, r in zip(names, got, ref)
+                  if n != "dx"}
+        parity = {k: float(f"{v:.3e}") for k, v in parity.items()}
+
+    out = {
+        "metric": "moe_layer_fwd_bwd_tokens_per_s", "value": round(tokens_per_s, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "full MoE layer fwd+bwd (gate, top-2 routing, fc1 ESMM+GELU, fc2 ESMM, ESS, ESTMM, "
+                               "backward ESMM), Swin-MoE-S stage-3 shape",
+                   "tokens": T, "d": D, "h": H, "experts": E, "top_k": K_TOP, "seed": SEED,
+                   "routing": "top-2 of softmax(x.wg + N(0,0.5) per-expert bias)"},
+        "tflops": round(flops_step / (ms * 1e-3) / 1e12, 1),
+        "frac_bf16_mfma_peak": round(flops_step / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+        "roofline": roofline, "cpu_baseline": cpu, "parity_rel_err_vs_cpu": parity, "kernels": kernels,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -29,6 +29,41 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+class OpTimer:
+    """Optional per-call device timing: while installed (set_timer), every operator call is bracketed
+    by two events on the stream it launches on.  durations() waits for the device."""
+
+    def __init__(self):
+        self.records = []
+
+    def durations(self):
+        torch.cuda.synchronize()
+        out = {}
+        for label, a, b in self.records:
+            out.setdefault(label, []).append(a.elapsed_time(b))  # ms
+        return out
+
+
+_timer = None
+
+
+def set_timer(timer):
+    global _timer
+    _timer = timer
+
+
+def _call(label, fn, *args):
+    if _timer is None:
+        return fn(*args)
+    a = torch.cuda.Event(enable_timing=True)
+    b = torch.cuda.Event(enable_timing=True)
+    a.record()
+    rc = fn(*args)
+    b.record()
+    _timer.records.append((label, a, b))
+    return rc
+
+
 class Route:
     """Routing metadata of one MoE depth: a view of a caller-owned int32 blob (see
     hexa_route_layout in include/hexa_moe_hip.h)."""
@@ -93,8 +128,8 @@ def route_build(routing, num_experts, blob=None):
     T, k = routing.shape
     if blob is None:
         blob = torch.empty(max(route_blob_ints(T, k, num_experts), 4), dtype=torch.int32, device=routing.device)
-    rc = _lib.load().hexa_route_build(_ptr(routing), int(routing.dtype == torch.int64), routing.stride(0),
-                                      routing.stride(1), T, k, num_experts, _ptr(blob), _stream())
+    rc = _call("route_build", _lib.load().hexa_route_build, _ptr(routing), int(routing.dtype == torch.int64),
+               routing.stride(0), routing.stride(1), T, k, num_experts, _ptr(blob), _stream())
     _lib.check(rc, "hexa_route_build")
     return Route(blob, T, k, num_experts)
 
@@ -129,10 +164,12 @@ def esmm(x, w, bias, route, m2s, w_layout, out=None, out_dtype=None, accumulate=
     out_act = torch.empty_like(out) if gelu else None
     if bias is not None:
         bias = bias.contiguous()
-    rc = _lib.load().hexa_esmm(_ptr(out), _ptr(x), _ptr(w), _ptr(bias), _ptr(route.blob), int(bool(m2s)),
-                               int(w_layout), int(bool(accumulate)), T, k, in_dim, out_dim, E, _dt(x), _dt(w),
-                               _dt(bias) if bias is not None else 0, _dt(out),
-                               _lib.HEXA_ACT_GELU if gelu else _lib.HEXA_ACT_NONE, _ptr(out_act), _stream())
+    label = f"esmm[{in_dim}->{out_dim},{'w_in_out' if w_layout == _lib.HEXA_W_IN_OUT else 'w_out_in'}" \
+            f"{',sum_slots' if m2s else ''}{',gelu' if gelu else ''}]"
+    rc = _call(label, _lib.load().hexa_esmm, _ptr(out), _ptr(x), _ptr(w), _ptr(bias), _ptr(route.blob),
+               int(bool(m2s)), int(w_layout), int(bool(accumulate)), T, k, in_dim, out_dim, E, _dt(x), _dt(w),
+               _dt(bias) if bias is not None else 0, _dt(out),
+               _lib.HEXA_ACT_GELU if gelu else _lib.HEXA_ACT_NONE, _ptr(out_act), _stream())
     _lib.check(rc, "hexa_esmm")
     return (out, out_act) if gelu else out
 
@@ -150,9 +187,9 @@ def estmm(dy, x, route, dy_per_slot, x_per_slot, out=None, out_dtype=torch.float
     if out is None:
         assert not accumulate
         out = torch.empty(E, out_dim, in_dim, dtype=out_dtype, device=x.device)
-    rc = _lib.load().hexa_estmm(_ptr(out), _ptr(dy), _ptr(x), _ptr(route.blob), int(bool(dy_per_slot)),
-                                int(bool(x_per_slot)), int(bool(accumulate)), T, k, out_dim, in_dim, E, _dt(x),
-                                _dt(out), _stream())
+    rc = _call(f"estmm[{out_dim}x{in_dim}]", _lib.load().hexa_estmm, _ptr(out), _ptr(dy), _ptr(x), _ptr(route.blob),
+               int(bool(dy_per_slot)), int(bool(x_per_slot)), int(bool(accumulate)), T, k, out_dim, in_dim, E,
+               _dt(x), _dt(out), _stream())
     _lib.check(rc, "hexa_estmm")
     return out
 
@@ -167,8 +204,9 @@ def ess(dy, route, dy_per_slot, out=None, out_dtype=torch.float32, accumulate=Fa
     if out is None:
         assert not accumulate
         out = torch.empty(E, out_dim, dtype=out_dtype, device=dy.device)
-    rc = _lib.load().hexa_ess(_ptr(out), _ptr(dy), _ptr(route.blob), int(bool(dy_per_slot)), int(bool(accumulate)),
-                              T, k, out_dim, E, _dt(dy), _dt(out), _stream())
+    rc = _call(f"ess[{out_dim}{',per_slot' if dy_per_slot else ''}]", _lib.load().hexa_ess, _ptr(out), _ptr(dy),
+               _ptr(route.blob), int(bool(dy_per_slot)), int(bool(accumulate)), T, k, out_dim, E, _dt(dy), _dt(out),
+               _stream())
     _lib.check(rc, "hexa_ess")
     return out
 
@@ -180,6 +218,7 @@ def gelu_bwd(dy2, y1):
     y1 = y1.contiguous()
     assert dy2.shape == y1.shape and dy2.dtype == y1.dtype
     out = torch.empty_like(dy2)
-    rc = _lib.load().hexa_gelu_bwd(_ptr(out), _ptr(dy2), _ptr(y1), dy2.numel(), _dt(dy2), _stream())
+    rc = _call("gelu_bwd", _lib.load().hexa_gelu_bwd, _ptr(out), _ptr(dy2), _ptr(y1), dy2.numel(), _dt(dy2),
+               _stream())
     _lib.check(rc, "hexa_gelu_bwd")
     return out

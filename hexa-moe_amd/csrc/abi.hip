@@ -1,6 +1,7 @@
 // C ABI of libhexa_moe_hip.so (declared in include/hexa_moe_hip.h): argument validation, dtype
 // dispatch and error reporting around the kernel launchers.  Nothing here allocates device memory
 // or waits for the device.
+#include <stdlib.h>
 #include <string.h>
 
 #include "hexa_internal.h"
@@ -14,6 +15,12 @@ void set_error(const char* fmt, ...) {
     va_start(ap, fmt);
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
+}
+
+// HEXA_MOE_GENERAL_KERNELS=1 forces the general kernels (testing aid; read once).
+bool dma_path_enabled() {
+    static const bool on = [] { const char* v = getenv("HEXA_MOE_GENERAL_KERNELS"); return !(v && v[0] == '1'); }();
+    return on;
 }
 
 static bool is_dt(int dt) { return dt == HEXA_F32 || dt == HEXA_F16 || dt == HEXA_BF16; }
@@ -64,6 +71,7 @@ extern "C" int hexa_esmm(void* out, const void* x, const void* w, const void* bi
         HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_esmm: result must be fp32 or the tokens' 16-bit type");
     if (bias && bias_dt != x_dt && bias_dt != HEXA_F32)
         HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_esmm: bias must be fp32 or the tokens' 16-bit type");
+    if (dma_path_enabled() && esmm16_dma_supported(a)) return launch_esmm16_dma(a, st);
     return launch_esmm16(a, st);
 }
 
@@ -82,6 +90,7 @@ extern "C" int hexa_estmm(void* dw, const void* dy, const void* x, const int32_t
     a.m_dim = out_dim; a.n_dim = in_dim;
     a.p_per_slot = dy_per_slot ? 1 : 0; a.q_per_slot = x_per_slot ? 1 : 0;
     a.accumulate = accumulate ? 1 : 0; a.pq_dt = dt; a.dw_dt = dw_dt;
+    if (is_16(dt) && dma_path_enabled() && estmm16_dma_supported(a)) return launch_estmm16_dma(a, st);
     return is_16(dt) ? launch_estmm16(a, st) : launch_estmm32(a, st);
 }
 

@@ -71,6 +71,11 @@ struct EssArgs {
 
 int launch_esmm16(const EsmmArgs& a, hipStream_t s);
 int launch_esmm32(const EsmmArgs& a, hipStream_t s);
+bool esmm16_dma_supported(const EsmmArgs& a);
+int launch_esmm16_dma(const EsmmArgs& a, hipStream_t s);
+bool dma_path_enabled();
+bool estmm16_dma_supported(const EstmmArgs& a);
+int launch_estmm16_dma(const EstmmArgs& a, hipStream_t s);
 int launch_estmm16(const EstmmArgs& a, hipStream_t s);
 int launch_estmm32(const EstmmArgs& a, hipStream_t s);
 int launch_ess(const EssArgs& a, hipStream_t s);

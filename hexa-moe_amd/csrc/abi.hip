@@ -41,7 +41,8 @@ extern "C" int hexa_abi_version(void) { return HEXA_ABI_VERSION; }
 
 extern "C" int hexa_esmm(void* out, const void* x, const void* w, const void* bias, const int32_t* route, int m2s,
                          int w_layout, int accumulate, int T, int k, int in_dim, int out_dim, int E, int x_dt,
-                         int w_dt, int bias_dt, int out_dt, int act, void* out_act, void* stream) {
+                         int w_dt, int bias_dt, int out_dt, int act, void* out_act, void* slot_ws,
+                         void* stream) {
     if (int rc = check_sizes("hexa_esmm", T, k, E, in_dim, out_dim)) return rc;
     if (!out || !x || !w || !route) HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: null pointer");
     if (w_layout != HEXA_W_IN_OUT && w_layout != HEXA_W_OUT_IN) HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: bad w_layout %d", w_layout);
@@ -52,7 +53,7 @@ extern "C" int hexa_esmm(void* out, const void* x, const void* w, const void* bi
         HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: a fused activation needs out_act, m2s == 0 and accumulate == 0");
     if (T == 0) return HEXA_OK;
     EsmmArgs a;
-    a.out = out; a.x = x; a.w = w; a.bias = bias; a.out_act = out_act;
+    a.out = out; a.x = x; a.w = w; a.bias = bias; a.out_act = out_act; a.slot_ws = slot_ws;
     a.r = route_view(route, T, k, E);
     a.in_dim = in_dim; a.out_dim = out_dim;
     a.x_per_slot = m2s ? 1 : 0;
@@ -110,12 +111,13 @@ extern "C" int hexa_ess(void* db, const void* dy, const int32_t* route, int dy_p
 
 extern "C" int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y, const void* w, const void* x,
                                const int32_t* route, int m2s, int accumulate, int T, int k, int in_dim, int out_dim,
-                               int E, int act_dt, int w_dt, int jx_dt, int jw_dt, int jb_dt, void* stream) {
+                               int E, int act_dt, int w_dt, int jx_dt, int jw_dt, int jb_dt, void* slot_ws,
+                               void* stream) {
     if (!j_x || !j_w || !j_y || !w || !x || !route) HEXA_FAIL(HEXA_ERR_ARG, "hexa_fused_grad: null pointer");
     // ESMM task: j_x = j_y . w[e] with w [E][out][in] read as an [E][in'=out][out'=in] weight; the
     // slot layout is the mirror image of the forward's (shared j_y -> per-slot j_x and vice versa).
     int rc = hexa_esmm(j_x, j_y, w, nullptr, route, m2s, HEXA_W_IN_OUT, accumulate, T, k, out_dim, in_dim, E, act_dt,
-                       w_dt, HEXA_F32, jx_dt, HEXA_ACT_NONE, nullptr, stream);
+                       w_dt, HEXA_F32, jx_dt, HEXA_ACT_NONE, nullptr, slot_ws, stream);
     if (rc) return rc;
     // ESTMM task: j_w[e][out][in] = sum j_y^T x
     rc = hexa_estmm(j_w, j_y, x, route, m2s ? 1 : 0, m2s ? 0 : 1, accumulate, T, k, out_dim, in_dim, E, act_dt, jw_dt,

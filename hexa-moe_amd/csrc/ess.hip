@@ -29,6 +29,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void ess_kernel(EssK p) {
     constexpr int V = Vec16<T>::N;
     constexpr int STRIP = 8 * V;  // columns per workgroup
+    constexpr int U = 8;          // rows in flight per lane: 256 rows (32 KiB) per workgroup step
     __shared__ float red[4][STRIP];
     const int e = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -48,21 +49,22 @@ __global__ __launch_bounds__(256) void ess_kernel(EssK p) {
         any = any || end > beg;
         const int32_t* tok = p.token_ids + (size_t)s * p.T;
         const T* base = dy + (size_t)p.dy_slot_rows * s * p.N + col;
-        // 32 rows per workgroup step, 4 steps in flight
-        for (int r0 = beg + wave * 8 + rg; r0 < end; r0 += 128) {
-            union { uint4 u; T e[V]; } v[4];
+        // this lane's rows: beg + wave*8 + rg + 32*u + 256*step; the token ids of the next step are
+        // fetched while the rows of the current one are in flight
+        const int r_lane = beg + wave * 8 + rg;
+        int ids[U];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int r = r0 + 32 * u;
-                if (r < end && col_ok) {
-                    const int t = tok[r];
-                    v[u].u = *reinterpret_cast<const uint4*>(base + (size_t)t * p.N);
-                } else {
-                    v[u].u = make_uint4(0u, 0u, 0u, 0u);
-                }
-            }
+        for (int u = 0; u < U; ++u) { const int r = r_lane + 32 * u; ids[u] = r < end ? tok[r] : -1; }
+        for (int r0 = r_lane; r0 < end; r0 += 32 * U) {
+            union { uint4 u; T e[V]; } v[U];
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+            for (int u = 0; u < U; ++u)
+                v[u].u = (ids[u] >= 0 && col_ok) ? *reinterpret_cast<const uint4*>(base + (size_t)ids[u] * p.N)
+                                                 : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+            for (int u = 0; u < U; ++u) { const int r = r0 + 32 * U + 32 * u; ids[u] = r < end ? tok[r] : -1; }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
 #pragma unroll
                 for (int i = 0; i < V; ++i) acc[i] += Cvt<T>::to_f(v[u].e[i]);
         }
@@ -146,7 +148,49 @@ int launch_gelu_bwd_t(void* dy1, const void* dy2, const void* y1, int64_t n, hip
     return HEXA_OK;
 }
 
+// out[i] += ws[0][i] + ws[1][i] + ... in fp32, slot order (the deterministic reduction behind the
+// one-launch slot sum of ESMM)
+template <typename T>
+__global__ __launch_bounds__(256) void sum_slots_kernel(T* __restrict__ out, const T* __restrict__ ws, int64_t n,
+                                                        int nws) {
+    constexpr int V = Vec16<T>::N;
+    const int64_t nv = n / V;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nv; i += stride) {
+        union { uint4 u; T e[V]; } o, w;
+        o.u = reinterpret_cast<const uint4*>(out)[i];
+        float acc[V];
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc[j] = Cvt<T>::to_f(o.e[j]);
+        for (int s = 0; s < nws; ++s) {
+            w.u = reinterpret_cast<const uint4*>(ws + (size_t)s * n)[i];
+#pragma unroll
+            for (int j = 0; j < V; ++j) acc[j] += Cvt<T>::to_f(w.e[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < V; ++j) o.e[j] = Cvt<T>::from_f(acc[j]);
+        reinterpret_cast<uint4*>(out)[i] = o.u;
+    }
+}
+
+template <typename T>
+int launch_sum_slots_t(void* out, const void* ws, int64_t n, int nws, hipStream_t st) {
+    if (n == 0 || nws == 0) return HEXA_OK;
+    if (n % Vec16<T>::N) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "sum_slots: size must be a multiple of the vector width");
+    int64_t blocks = (n / Vec16<T>::N + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    hipLaunchKernelGGL((sum_slots_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, (T*)out, (const T*)ws, n, nws);
+    HEXA_CHECK_LAUNCH("sum_slots");
+    return HEXA_OK;
+}
+
 }  // namespace
+
+int launch_sum_slots(void* out, const void* ws, int64_t n, int nws, int dt, hipStream_t st) {
+    if (dt == HEXA_F32) return launch_sum_slots_t<float>(out, ws, n, nws, st);
+    if (dt == HEXA_BF16) return launch_sum_slots_t<__bf16>(out, ws, n, nws, st);
+    return launch_sum_slots_t<_Float16>(out, ws, n, nws, st);
+}
 
 int launch_ess(const EssArgs& a, hipStream_t st) {
     if (a.dy_dt == HEXA_F32) return launch_ess_t<float>(a, st);

@@ -126,7 +126,7 @@ __device__ __forceinline__ V frag_ks(const char* tile, int col0, int ks, int lan
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
         const int kk = k + half * 4;
-        const int pos = ch ^ ((kk & 7) << 1);
+        const int pos = ch ^ ((kk & 3) << 2);
         r.h[half] = lds_read_tr16(base + kk * 256 + pos * 16 + sub);
     }
     return r.v;
@@ -202,6 +202,7 @@ struct EsmmK {
     int x_slot_rows, out_slot_rows;
     int accumulate, bias_dt, out_dt, act, group;
     long total;
+    void* ws;   // slots > 0 write here ([slot-1][T][N]) when set: the slots are summed afterwards
 };
 
 template <typename TC, bool W_IN_OUT, bool OUT32>
@@ -243,7 +244,7 @@ __global__ __launch_bounds__(NT, 2) void esmm16_dma_kernel(EsmmK p) {
         }
         if (W_IN_OUT) {  // w[e][k][n], KS: chunk covers k rows 4*chunk .. +3, 16 pieces of 8 columns
             const int kk = 4 * (wave + 4 * c) + (lane >> 4);
-            const int ch = (lane & 15) ^ ((kk & 7) << 1);
+            const int ch = (lane & 15) ^ ((kk & 3) << 2);
             const int n = n0 + ch * 8;
             const bool ok = n < N;
             srcB[c] = ok ? reinterpret_cast<const char*>(p.w) + (((size_t)e * K + kk) * N + n) * 2 : zero;
@@ -288,9 +289,11 @@ __global__ __launch_bounds__(NT, 2) void esmm16_dma_kernel(EsmmK p) {
     }
 
     // ---- epilogue: lane holds, per 32x32 block, token row l%32 and 4 consecutive columns per group ----
-    const bool accumulate = p.accumulate != 0;
+    const bool to_ws = p.ws != nullptr && s > 0;
+    void* const outp = to_ws ? p.ws : p.out;
+    const bool accumulate = p.accumulate != 0 && !to_ws;
     const bool gelu = p.act == HEXA_ACT_GELU;
-    const size_t out_base = (size_t)p.out_slot_rows * s;
+    const size_t out_base = to_ws ? (size_t)p.T * (s - 1) : (size_t)p.out_slot_rows * s;
     constexpr int CP = BN * 2 + 16;  // pitch (bytes) of the staged 16-bit result tile
     if (!OUT32) barrier_nofence();   // the stage buffers are reused for the result tile
 #pragma unroll
@@ -320,7 +323,7 @@ __global__ __launch_bounds__(NT, 2) void esmm16_dma_kernel(EsmmK p) {
                     const int tok = sTok[rl];
                     if (tok < 0 || n >= N) continue;
                     const size_t off = (out_base + tok) * N + n;
-                    float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(p.out) + off);
+                    float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(outp) + off);
                     if (accumulate) { const float4 old = *dst; v[0] += old.x; v[1] += old.y; v[2] += old.z; v[3] += old.w; }
                     *dst = make_float4(v[0], v[1], v[2], v[3]);
                     if (gelu)
@@ -344,7 +347,7 @@ __global__ __launch_bounds__(NT, 2) void esmm16_dma_kernel(EsmmK p) {
                 if (tok < 0) continue;
                 const size_t off = (out_base + tok) * N + n;
                 uint4 val = *reinterpret_cast<const uint4*>(smem + rl * CP + c * 16);
-                uint4* dst = reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(p.out) + off);
+                uint4* dst = reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(outp) + off);
                 if (accumulate) {
                     const uint4 old = *dst;
                     const unsigned ow[4] = {old.x, old.y, old.z, old.w};
@@ -375,12 +378,12 @@ __global__ __launch_bounds__(NT, 2) void esmm16_dma_kernel(EsmmK p) {
 
 int round_up(long v, int m) { return (int)(((v + m - 1) / m) * m); }
 
-template <typename K> int ensure_smem(K kernel) {
+template <typename K> int ensure_smem(K kernel, int bytes) {
     static bool done = false;  // per instantiation
     if (!done) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                SMEM_BYTES) != hipSuccess)
-            HEXA_FAIL(HEXA_ERR_LAUNCH, "hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d) failed", SMEM_BYTES);
+                                bytes) != hipSuccess)
+            HEXA_FAIL(HEXA_ERR_LAUNCH, "hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d) failed", bytes);
         done = true;
     }
     return HEXA_OK;
@@ -389,7 +392,7 @@ template <typename K> int ensure_smem(K kernel) {
 template <typename TC, bool IO, bool OUT32>
 int launch_esmm_dma_t(EsmmK& p, int grid, hipStream_t st) {
     auto kernel = esmm16_dma_kernel<TC, IO, OUT32>;
-    if (int rc = ensure_smem(kernel)) return rc;
+    if (int rc = ensure_smem(kernel, SMEM_BYTES)) return rc;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), SMEM_BYTES, st, p);
     HEXA_CHECK_LAUNCH("esmm16_dma");
     return HEXA_OK;
@@ -400,6 +403,9 @@ int launch_esmm_dma_t(EsmmK& p, int grid, hipStream_t st) {
 // ------------------------------------------------------------------------------------------------
 constexpr int MAX_SLOTS = 8;      // routing slots handled by this path
 constexpr int TOK_RING = 8;       // steps of token ids kept in LDS (32 ids each)
+constexpr int ESTMM_STAGE_AREA = 128 * (BN + 4) * 4;   // >= STAGES * STAGE_BYTES: also holds the staged fp32 result
+constexpr int ESTMM_SMEM_BYTES = ESTMM_STAGE_AREA + TOK_RING * 32 * 4;
+static_assert(ESTMM_STAGE_AREA >= STAGES * STAGE_BYTES, "result staging must cover the stage buffers");
 
 struct EstmmK {
     const void* pm; const void* qm; void* dw;
@@ -417,19 +423,44 @@ struct Cursor {   // walks the expert's token list in 32-token steps, slot after
 template <typename TC, bool OUT32>
 __global__ __launch_bounds__(NT, 2) void estmm16_dma_kernel(EstmmK p) {
     extern __shared__ __attribute__((aligned(1024))) char smem[];
-    int* sIds = reinterpret_cast<int*>(smem + STAGES * STAGE_BYTES);   // [TOK_RING][32]
+    int* sIds = reinterpret_cast<int*>(smem + ESTMM_STAGE_AREA);       // [TOK_RING][32]
     __shared__ int sBeg[MAX_SLOTS], sEnd[MAX_SLOTS];
 
+    __shared__ int sExpert;
     const long logical = logical_tile(p.group);
     if (logical >= p.total) return;
     const int per_e = p.mtn * p.ntn;
-    const int e = (int)(logical / per_e);
-    const int rem = (int)(logical - (long)e * per_e);
+    const int rank = (int)(logical / per_e);
+    const int rem = (int)(logical - (long)rank * per_e);
     const int m0 = (rem / p.ntn) * BM, n0 = (rem % p.ntn) * BN;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wr = wave >> 1, wf = wave & 1;
     const int M = p.M, N = p.N, T = p.T, nslot = p.k;
+
+    // Heaviest experts first: workgroups are dispatched in id order, so giving the long token lists
+    // to the first ones shortens the tail.  The expert of this workgroup is the one whose load has
+    // rank `rank` (ties broken by index).  Up to 256 experts; beyond that the order is by index.
+    int e = rank;
+    if (p.E <= NT) {
+        auto load_of = [&](int x) {
+            int t = 0;
+            for (int s = 0; s < nslot; ++s)
+                t += p.offsets[(size_t)s * (p.E + 1) + x + 1] - p.offsets[(size_t)s * (p.E + 1) + x];
+            return t;
+        };
+        if (tid < p.E) {
+            const int mine = load_of(tid);
+            int r = 0;
+            for (int x = 0; x < p.E; ++x) {
+                const int o = load_of(x);
+                r += (o > mine || (o == mine && x < tid)) ? 1 : 0;
+            }
+            if (r == rank) sExpert = tid;
+        }
+        __syncthreads();
+        e = sExpert;
+    }
 
     if (tid < nslot) {
         sBeg[tid] = p.offsets[(size_t)tid * (p.E + 1) + e];
@@ -472,7 +503,7 @@ __global__ __launch_bounds__(NT, 2) void estmm16_dma_kernel(EstmmK p) {
 #pragma unroll
         for (int cc = 0; cc < 2; ++cc) {
             const int kk = 4 * (wave + 4 * cc) + (lane >> 4);
-            const int ch = ch0 ^ ((kk & 7) << 1);
+            const int ch = ch0 ^ ((kk & 3) << 2);
             const bool row_ok = c.r + kk < end;
             const int tok = toks[cc];
             const bool okp = row_ok && (m0 + ch * 8 < M), okq = row_ok && (n0 + ch * 8 < N);
@@ -520,45 +551,59 @@ __global__ __launch_bounds__(NT, 2) void estmm16_dma_kernel(EstmmK p) {
     }
 
     // ---- epilogue: lane holds row m = l%32 of a block and 4 consecutive n per group ----
+    // The block leaves through LDS (pitch 132 floats) so that 32 lanes write one contiguous 512-byte
+    // row of dw; 16-bit results are packed on the way out.
     const bool accumulate = p.accumulate != 0;
+    constexpr int CPF = BN + 4;   // floats per staged row
+    float* sC = reinterpret_cast<float*>(smem);
+    barrier_nofence();            // all wavefronts are done reading the stage buffers
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        const int m = m0 + wr * 64 + i * 32 + (lane & 31);
-        if (m >= M) continue;
+        const int ml = wr * 64 + i * 32 + (lane & 31);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const int n = n0 + wf * 64 + j * 32 + 8 * g + 4 * (lane >> 5);
-                if (n >= N) continue;
+                const int nl = wf * 64 + j * 32 + 8 * g + 4 * (lane >> 5);
+                *reinterpret_cast<float4*>(sC + ml * CPF + nl) =
+                    make_float4(acc[j][i][4 * g], acc[j][i][4 * g + 1], acc[j][i][4 * g + 2], acc[j][i][4 * g + 3]);
+            }
+        }
+    }
+    __syncthreads();
+    {
+        const int c = tid & 31, n = n0 + c * 4;
+        if (n < N) {
+#pragma unroll 4
+            for (int it = 0; it < BM / 8; ++it) {
+                const int ml = it * 8 + (tid >> 5);
+                const int m = m0 + ml;
+                if (m >= M) break;
+                float4 v = *reinterpret_cast<const float4*>(sC + ml * CPF + c * 4);
                 const size_t off = ((size_t)e * M + m) * N + n;
-                float v[4];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) v[q] = acc[j][i][4 * g + q];
                 if (OUT32) {
                     float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(p.dw) + off);
-                    if (accumulate) { const float4 old = *dst; v[0] += old.x; v[1] += old.y; v[2] += old.z; v[3] += old.w; }
-                    *dst = make_float4(v[0], v[1], v[2], v[3]);
+                    if (accumulate) { const float4 old = *dst; v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w; }
+                    *dst = v;
                 } else {
                     uint2* dst = reinterpret_cast<uint2*>(reinterpret_cast<unsigned short*>(p.dw) + off);
                     if (accumulate) {
                         const uint2 old = *dst;
-                        v[0] += from_bits16<TC>(old.x & 0xffff); v[1] += from_bits16<TC>(old.x >> 16);
-                        v[2] += from_bits16<TC>(old.y & 0xffff); v[3] += from_bits16<TC>(old.y >> 16);
+                        v.x += from_bits16<TC>(old.x & 0xffff); v.y += from_bits16<TC>(old.x >> 16);
+                        v.z += from_bits16<TC>(old.y & 0xffff); v.w += from_bits16<TC>(old.y >> 16);
                     }
-                    *dst = pack4<TC>(v[0], v[1], v[2], v[3]);
+                    *dst = pack4<TC>(v.x, v.y, v.z, v.w);
                 }
             }
         }
     }
 }
 
-constexpr int ESTMM_SMEM_BYTES = STAGES * STAGE_BYTES + TOK_RING * 32 * 4;
 
 template <typename TC, bool OUT32>
 int launch_estmm_dma_t(EstmmK& p, int grid, hipStream_t st) {
     auto kernel = estmm16_dma_kernel<TC, OUT32>;
-    if (int rc = ensure_smem(kernel)) return rc;
+    if (int rc = ensure_smem(kernel, ESTMM_SMEM_BYTES)) return rc;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), ESTMM_SMEM_BYTES, st, p);
     HEXA_CHECK_LAUNCH("estmm16_dma");
     return HEXA_OK;
@@ -603,10 +648,15 @@ int launch_esmm16_dma(const EsmmArgs& a, hipStream_t st) {
     p.out_slot_rows = a.out_per_slot ? a.r.T : 0;
     p.bias_dt = a.bias_dt; p.out_dt = a.out_dt; p.act = a.act;
     p.group = p.ntn * 4;
-    const int launches = a.out_per_slot ? 1 : a.r.k;
+    // Summing the slots into one result: with scratch, every slot runs in ONE launch (slot 0 into
+    // `out`, the others into the scratch) and a reduction adds them in slot order; without it, one
+    // launch per slot, each adding into `out`.
+    const bool one_launch = a.out_per_slot || a.r.k == 1 || a.slot_ws != nullptr;
+    p.ws = (!a.out_per_slot && a.r.k > 1) ? a.slot_ws : nullptr;
+    const int launches = one_launch ? 1 : a.r.k;
     for (int l = 0; l < launches; ++l) {
-        p.slot_begin = a.out_per_slot ? 0 : l;
-        p.nslots = a.out_per_slot ? a.r.k : 1;
+        p.slot_begin = one_launch ? 0 : l;
+        p.nslots = one_launch ? a.r.k : 1;
         p.accumulate = (a.accumulate || l > 0) ? 1 : 0;
         p.total = (long)p.nslots * p.mt_ub * p.ntn;
         if (p.total == 0) continue;
@@ -623,6 +673,7 @@ int launch_esmm16_dma(const EsmmArgs& a, hipStream_t st) {
         }
         if (rc) return rc;
     }
+    if (p.ws) return launch_sum_slots(a.out, a.slot_ws, (int64_t)a.r.T * a.out_dim, a.r.k - 1, a.out_dt, st);
     return HEXA_OK;
 }
 

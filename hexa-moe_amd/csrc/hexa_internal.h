@@ -46,7 +46,7 @@ RouteView route_view(const int32_t* route, int T, int k, int E);
 
 // ---- launchers implemented in the kernel files ----------------------------------------------
 struct EsmmArgs {
-    void* out; const void* x; const void* w; const void* bias; void* out_act;
+    void* out; const void* x; const void* w; const void* bias; void* out_act; void* slot_ws;
     RouteView r;
     int in_dim, out_dim;
     int x_per_slot, out_per_slot;  // row operand / result indexed [slot][T][*] (1) or [T][*] (0)
@@ -79,6 +79,7 @@ int launch_estmm16_dma(const EstmmArgs& a, hipStream_t s);
 int launch_estmm16(const EstmmArgs& a, hipStream_t s);
 int launch_estmm32(const EstmmArgs& a, hipStream_t s);
 int launch_ess(const EssArgs& a, hipStream_t s);
+int launch_sum_slots(void* out, const void* ws, int64_t n, int nws, int dt, hipStream_t s);
 int launch_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, hipStream_t s);
 
 // ---- small device helpers -------------------------------------------------------------------

@@ -31,10 +31,10 @@ SIGNATURES = {
     "hexa_token_count": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "hexa_token_assign": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "hexa_route_from_lists": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
-    "hexa_esmm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
+    "hexa_esmm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "hexa_estmm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "hexa_ess": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
-    "hexa_fused_grad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "hexa_fused_grad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "hexa_gelu_bwd": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),
     "hexa_last_error": (ctypes.c_char_p, []),
     "hexa_abi_version": (_i, []),
@@ -57,7 +57,7 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.hexa_abi_version() != 1:
+    if lib.hexa_abi_version() != 2:
         raise RuntimeError("hexa_moe: libhexa_moe_hip.so has an unexpected ABI version")
     _lib = lib
     return lib

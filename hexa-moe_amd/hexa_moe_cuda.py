@@ -100,10 +100,12 @@ def _fused(j_b, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, m2s, num_t
         ops._dev(t)
         if not t.is_contiguous():
             raise TypeError("FUSED_GRAD: tensors must be contiguous")
+    ws = torch.empty((k - 1) * T * int(num_in_dims), dtype=j_x.dtype, device=j_x.device) if (m2s and k > 1) else None
     rc = _lib.load().hexa_fused_grad(
         j_b.data_ptr() if j_b is not None else None, j_x.data_ptr(), j_w.data_ptr(), j_y.data_ptr(), w.data_ptr(),
         x.data_ptr(), route.blob.data_ptr(), int(bool(m2s)), 1, T, k, int(num_in_dims), int(num_out_dims), E,
-        ops._dt(j_y), ops._dt(w), ops._dt(j_x), ops._dt(j_w), ops._dt(j_b) if j_b is not None else 0, ops._stream())
+        ops._dt(j_y), ops._dt(w), ops._dt(j_x), ops._dt(j_w), ops._dt(j_b) if j_b is not None else 0,
+        ws.data_ptr() if ws is not None else None, ops._stream())
     _lib.check(rc, "FUSED_GRAD")
 
 

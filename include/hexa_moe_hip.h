@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define HEXA_ABI_VERSION 1
+#define HEXA_ABI_VERSION 2
 
 /* element types */
 #define HEXA_F32 0
@@ -106,13 +106,17 @@ int hexa_route_from_lists(const int32_t* token_idx_list, const int32_t* expert_i
  * fp32 accumulation; out may be that 16-bit type or F32).  accumulate != 0 adds into `out`.
  * act == HEXA_ACT_GELU additionally writes gelu(out) to out_act (same shape/dtype as out; m2s == 0).
  * Dimension granularity: in and out multiples of 8 (16-bit) / 4 (fp32).
+ * slot_ws (may be NULL) is scratch for m2s != 0 with top_k > 1: (top_k-1)*T*out elements of out_dt.
+ * With it, all slots run in ONE launch (slot 0 writes `out`, the others write slot_ws) followed by a
+ * small reduction out += sum(slot_ws) in slot order; without it the slots run one launch after the
+ * other, each adding into `out`.  Both orders are fixed, so results are reproducible either way.
  * Replaces ESMM_TENSOR_CORE (torch/hexa_moe_ops.cpp:45-117) -> launch_esmm_accum_shared_tensor_{full,
  * mix,half} (include/hexa_moe.h:22-72, kernels/esmm_full.cu:249-300), and with w_layout OUT_IN the
  * ESMM task of FUSED_GRAD (kernels/fused_ops_full.cu:117-247). */
 int hexa_esmm(void* out, const void* x, const void* w, const void* bias, const int32_t* route, int m2s,
               int w_layout, int accumulate, int num_tokens, int top_k, int in_dim, int out_dim,
               int num_experts, int x_dt, int w_dt, int bias_dt, int out_dt, int act, void* out_act,
-              void* stream);
+              void* slot_ws, void* stream);
 
 /* ESTMM: dw[e][o][i] (+)= sum over slots s and tokens t routed to e of dy[(s),t,o] * x[(s),t,i].
  * dy_per_slot / x_per_slot say whether the operand is [k,T,*] (1) or [T,*] shared by the slots (0).
@@ -135,12 +139,13 @@ int hexa_ess(void* db, const void* dy, const int32_t* route, int dy_per_slot, in
  *   m2s == 0: j_y [T,out] shared, x and j_x [k,T,in]     (fc2 call, impls/layers.py:409-416)
  *   m2s != 0: j_y [k,T,out], x [T,in] shared, j_x [T,in] (fc1 call, impls/layers.py:435-451)
  * act_dt: element type of j_y and x; w_dt: of w; jx_dt / jw_dt / jb_dt: of the results.
+ * slot_ws: scratch of hexa_esmm for the m2s != 0 case ((top_k-1)*T*in elements of jx_dt) or NULL.
  * Replaces FUSED_GRAD / FUSED_GRAD_NO_BIAS (torch/hexa_moe_ops.cpp:119-275) ->
  * launch_fused_grad_{bias,no_bias}_{full,mix,half} (include/hexa_moe.h:74-181). */
 int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y, const void* w, const void* x,
                     const int32_t* route, int m2s, int accumulate, int num_tokens, int top_k, int in_dim,
                     int out_dim, int num_experts, int act_dt, int w_dt, int jx_dt, int jw_dt, int jb_dt,
-                    void* stream);
+                    void* slot_ws, void* stream);
 
 /* Elementwise backward of the fused GELU: dy1 = dy2 * gelu'(y1), n elements of type dt.  The
  * reference evaluates act' with torch.autograd.functional.jacobian (impls/layers.py:281-283,427). */

@@ -120,7 +120,7 @@ def test_fused_grad(dev, dtype, m2s, T, d_in, d_out, E, k, skew):
     jy_d, w_d, x_d = jy.to(dev), w.to(dev), x.to(dev)  # kept alive: only raw pointers cross the C ABI
     rc = _lib.load().hexa_fused_grad(jb.data_ptr(), jx.data_ptr(), jw.data_ptr(), jy_d.data_ptr(),
                                      w_d.data_ptr(), x_d.data_ptr(), route.blob.data_ptr(), int(m2s), 1,
-                                     T, k, d_in, d_out, E, ops._dt(jy), ops._dt(w), 0, 0, 0,
+                                     T, k, d_in, d_out, E, ops._dt(jy), ops._dt(w), 0, 0, 0, None,
                                      torch.cuda.current_stream().cuda_stream)
     _lib.check(rc, "hexa_fused_grad")
     torch.cuda.synchronize()

@@ -33,13 +33,13 @@ def test_header_symbols_are_exported():
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in include/hexa_moe_hip.h but not exported"
     assert declared == set(_lib.SIGNATURES), "ctypes table and header disagree"
-    assert lib.hexa_abi_version() == 1
+    assert lib.hexa_abi_version() == 2
 
 
 def test_abi_argument_errors_without_a_gpu():
     from hexa_moe import _lib
     lib = _lib.load()
-    assert lib.hexa_esmm(None, None, None, None, None, 0, 0, 0, 16, 1, 8, 8, 2, 0, 0, 0, 0, 0, None, None) == -1
+    assert lib.hexa_esmm(None, None, None, None, None, 0, 0, 0, 16, 1, 8, 8, 2, 0, 0, 0, 0, 0, None, None, None) == -1
     assert b"null pointer" in lib.hexa_last_error()
     assert lib.hexa_route_layout_get(-1, 1, 1, ctypes.byref(_lib.RouteLayout())) == -1
     assert lib.hexa_token_count(None, None, None, 4, 2, 1, None, None) == -1

@@ -1,13 +1,18 @@
 // Fast path of ESMM and ESTMM for bf16 / fp16 on gfx950 (CDNA4): tiles stream from HBM straight into
 // LDS with the asynchronous global->LDS copy (global_load_lds_dwordx4, 16 bytes per lane, no VGPR
-// staging), four stages deep, and are fed to v_mfma_f32_32x32x16 with fp32 accumulation.
+// staging), several stages deep, and are fed to v_mfma_f32_32x32x16 with fp32 accumulation.
 //
-// LDS tile formats (one operand tile = 128 output rows x 32 contraction indices = 8 KiB per stage):
-//   KC  "contraction index fastest in memory"  [128 rows][32 k]  64 B per row; a wavefront copy
+// Workgroup tile: BM x BN with WR x WF wavefronts of 64x64 each.  Two shapes are instantiated:
+//   128 x 128 (4 wavefronts, 4 stages, 64 KiB LDS, 2 workgroups per CU)  -- small problems
+//   256 x 128 (8 wavefronts, 3 stages, 72 KiB LDS, 2 workgroups per CU)  -- a third less L2 traffic
+//   per flop; with 128x128 tiles these kernels sit on the L2 -> LDS bandwidth, not on the MFMA pipe.
+//
+// LDS tile formats (per stage an operand tile holds W output rows x 32 contraction indices):
+//   KC  "contraction index fastest in memory"  [W rows][32 k]  64 B per row; a wavefront copy
 //       (64 lanes x 16 B = 1 KiB, contiguous in LDS) covers 16 rows.  Fragments: ds_read_b128.
 //       Token rows of ESMM (gathered through the tile's token ids) and w[E][out][in].
-//   KS  "contraction index slowest in memory"   [32 k][128 rows] 256 B per k; a wavefront copy covers
-//       4 k.  Fragments: two ds_read_b64_tr_b16 (the CDNA4 transposing LDS read) per 32x16 fragment.
+//   KS  "contraction index slowest in memory"   [32 k][W rows] 2W B per k.  Fragments: two
+//       ds_read_b64_tr_b16 (the CDNA4 transposing LDS read) per 32x16 fragment.
 //       w[E][in][out] of ESMM, and both operands of ESTMM (token rows of dy and x, tokens contracted).
 // The copy engine places lane i at LDS offset 16*i, so bank conflicts are avoided by choosing WHICH
 // 16-byte piece each lane fetches (an XOR swizzle applied on the global-address side) instead of
@@ -16,20 +21,38 @@
 //
 // The MFMA operands are swapped with respect to the usual convention (A = the operand that supplies
 // the output's fastest dimension, B = the rows), so every lane ends up with 4 consecutive output
-// columns and stores them with one 8-byte (16-bit results) or 16-byte (fp32 results) store.
+// columns; results leave through LDS so that whole 256- / 512-byte row pieces are stored.
 //
 // Constraints of this path (anything else runs on the general kernels of gemm16.hip): operands and
 // weights of one 16-bit type, in_dim a multiple of 32 for ESMM, out/in dims multiples of 8.
+#include <stdlib.h>
+
 #include "hexa_internal.h"
 
 namespace hexa {
 namespace {
 
-constexpr int BM = 128, BN = 128, BK = 32, STAGES = 4;
-constexpr int NT = 256;
-constexpr int TILE_BYTES = 128 * BK * 2;             // one operand tile of one stage
-constexpr int STAGE_BYTES = 2 * TILE_BYTES;          // A tile + B tile
-constexpr int SMEM_BYTES = STAGES * STAGE_BYTES + BM * 4;
+constexpr int BK = 32;
+
+// WR x WF wavefronts, each computing RB x FB blocks of 32x32 (RB blocks along the rows, FB along the
+// fast output dimension).  MINW = wavefronts per SIMD the register budget is sized for.
+template <int WR_, int WF_, int RB_, int FB_, int STAGES_, int MINW_>
+struct Cfg {
+    static constexpr int WR = WR_, WF = WF_, RB = RB_, FB = FB_, NW = WR_ * WF_, NT = 64 * NW, MINW = MINW_;
+    static constexpr int BM = 32 * RB_ * WR_, BN = 32 * FB_ * WF_, STAGES = STAGES_;
+    static constexpr int R_BYTES = BM * BK * 2, F_BYTES = BN * BK * 2, STAGE_BYTES = R_BYTES + F_BYTES;
+    static constexpr int R_COPIES = BM / 16, F_COPIES = BN / 16;      // wavefront copies per stage
+    static constexpr int R_CPW = R_COPIES / NW, F_CPW = F_COPIES / NW, CPW = R_CPW + F_CPW;
+    static constexpr int STAGE_AREA = STAGES * STAGE_BYTES;
+    static_assert(R_COPIES % NW == 0 && F_COPIES % NW == 0, "copies must divide evenly over the wavefronts");
+    static_assert(STAGES >= 3 && STAGES <= 4, "3 or 4 stages");
+};
+using CfgS = Cfg<2, 2, 2, 2, 4, 2>;   // 128 x 128, 4 wavefronts of 64x64
+using CfgL = Cfg<4, 2, 2, 2, 3, 4>;   // 256 x 128, 8 wavefronts of 64x64
+using CfgM = Cfg<2, 2, 4, 2, 3, 2>;   // 256 x 128, 4 wavefronts of 128x64
+using CfgX = Cfg<2, 2, 4, 4, 3, 1>;   // 256 x 256, 4 wavefronts of 128x128
+using CfgX8 = Cfg<2, 4, 4, 2, 3, 2>;  // 256 x 256, 8 wavefronts of 128x64
+using CfgX16 = Cfg<4, 4, 2, 2, 3, 4>; // 256 x 256, 16 wavefronts of 64x64
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
@@ -63,6 +86,12 @@ __device__ __forceinline__ void dma16(const void* src, char* lds_base) {
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
+// `ahead` copy groups of G copies each may still be in flight (ahead <= MAXA)
+template <int G, int MAXA> __device__ __forceinline__ void wait_groups(int ahead) {
+    if (MAXA >= 2 && ahead >= 2) wait_vmcnt<2 * G>();
+    else if (ahead >= 1) wait_vmcnt<G>();
+    else wait_vmcnt<0>();
+}
 
 // Workgroup barrier WITHOUT the memory fence of __syncthreads(): the fence would wait for every
 // outstanding copy (vmcnt(0)) and drain the pipeline.  Ordering is by hand: copies are awaited with
@@ -73,6 +102,9 @@ __device__ __forceinline__ void barrier_nofence() {
     asm volatile("" ::: "memory");
 }
 
+// Workgroup -> logical tile.  Workgroup ids go round-robin over the 8 XCDs (each with its own L2),
+// so runs of `group` consecutive logical tiles (which share token rows and an expert's weights) are
+// kept on one XCD.
 __device__ __forceinline__ long logical_tile(int group) {
     const int bid = blockIdx.x;
     const int xcd = bid & 7, loc = bid >> 3;
@@ -89,6 +121,7 @@ __device__ __forceinline__ V frag_kc(const char* tile, int row0, int ks, int lan
     const int pos = kch ^ ((row >> 2) & 3);
     return *reinterpret_cast<const V*>(tile + row * 64 + pos * 16);
 }
+
 // LDS reads issued as inline assembly: the compiler cannot see that they touch LDS, so it does not
 // order them behind the asynchronous copies in flight (it would insert s_waitcnt vmcnt(0) and drain
 // the pipeline).  Ordering against the copies is done by hand (wait_vmcnt + barrier); the data
@@ -106,16 +139,11 @@ __device__ __forceinline__ int lds_read_i32(unsigned addr) {
     asm volatile("ds_read_b32 %0, %1" : "=v"(r) : "v"(addr));
     return r;
 }
-template <typename V> __device__ __forceinline__ void lds_fence(V& a, V& b, V& c, V& d) {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
-}
-__device__ __forceinline__ void lds_fence(int& a, int& b) {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b));
-}
 
-// KS tile: same fragment from a [k][128] tile through two transposing reads (4 k each).
-// NOT usable before lds_fence() has been applied to it.
-template <typename V>
+// KS tile of width W: the same fragment from a [k][W] tile through two transposing reads (4 k each).
+// Chunk c (8 columns, 16 bytes) of row k sits at position c ^ (4*(k&3)) of the row: the four rows a
+// transposing read touches land on different banks.  NOT usable before lds_fence() has been applied.
+template <typename V, int W>
 __device__ __forceinline__ V frag_ks(const char* tile, int col0, int ks, int lane) {
     const int grp = lane >> 4, s = lane & 15;
     const int col = col0 + (grp & 1) * 16 + (s & 3) * 4;           // 4 consecutive columns = 8 bytes
@@ -127,38 +155,62 @@ __device__ __forceinline__ V frag_ks(const char* tile, int col0, int ks, int lan
     for (int half = 0; half < 2; ++half) {
         const int kk = k + half * 4;
         const int pos = ch ^ ((kk & 3) << 2);
-        r.h[half] = lds_read_tr16(base + kk * 256 + pos * 16 + sub);
+        r.h[half] = lds_read_tr16(base + kk * (2 * W) + pos * 16 + sub);
     }
     return r.v;
 }
 
-__device__ __forceinline__ void zero_acc(f32x16 (&acc)[2][2]) {
+// ---- copy-source helpers: which global piece does this lane fetch for wavefront copy `c` ------------
+// KC operand: copy c covers tile rows 16c..16c+15.
+__device__ __forceinline__ void kc_lane(int c, int lane, int& row, int& kc) {
+    row = 16 * c + (lane >> 2);
+    kc = (lane & 3) ^ ((row >> 2) & 3);
+}
+// KS operand of width W: copy c covers 512/W k rows; returns the k row and the column piece.
+template <int W> __device__ __forceinline__ void ks_lane(int c, int lane, int& kk, int& ch) {
+    constexpr int PPR = W / 8;               // 16-byte pieces per k row
+    constexpr int RPC = 64 / PPR;            // k rows per wavefront copy
+    kk = RPC * c + lane / PPR;
+    ch = (lane % PPR) ^ ((kk & 3) << 2);
+}
+
+template <int A, int B> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[A][B]) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < A; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < B; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 }
 
 // acc[j][i]: j = 32-wide block of the fast output dimension (operand "F"), i = 32-row block ("R").
-template <typename TC, bool F_KS, bool R_KS>
+template <typename V, int NA, int NB> __device__ __forceinline__ void lds_fence_all(V (&a)[NA], V (&b)[NB]) {
+    // one s_waitcnt that every fragment "passes through" (see lds_fence)
+    if constexpr (NA == 2 && NB == 2) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]));
+    else if constexpr (NA == 2 && NB == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+    else if constexpr (NA == 4 && NB == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+    else static_assert(NA == 2 && NB == 2, "unsupported fragment counts");
+}
+
+template <typename TC, typename C, bool F_KS, bool R_KS>
 __device__ __forceinline__ void mma_stage(const char* tileR, const char* tileF, int wr, int wf, int lane,
-                                          f32x16 (&acc)[2][2]) {
+                                          f32x16 (&acc)[C::FB][C::RB]) {
     using V = typename Mfma<TC>::V;
+    constexpr int RW = 32 * C::RB, FW = 32 * C::FB;   // rows / columns per wavefront
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
-        V f[2], r[2];
+        V f[C::FB], r[C::RB];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            f[i] = F_KS ? frag_ks<V>(tileF, wf * 64 + i * 32, ks, lane) : frag_kc<V>(tileF, wf * 64 + i * 32, ks, lane);
-            r[i] = R_KS ? frag_ks<V>(tileR, wr * 64 + i * 32, ks, lane) : frag_kc<V>(tileR, wr * 64 + i * 32, ks, lane);
-        }
-        if (F_KS || R_KS) lds_fence(f[0], f[1], r[0], r[1]);
+        for (int j = 0; j < C::FB; ++j)
+            f[j] = F_KS ? frag_ks<V, C::BN>(tileF, wf * FW + j * 32, ks, lane) : frag_kc<V>(tileF, wf * FW + j * 32, ks, lane);
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int i = 0; i < C::RB; ++i)
+            r[i] = R_KS ? frag_ks<V, C::BM>(tileR, wr * RW + i * 32, ks, lane) : frag_kc<V>(tileR, wr * RW + i * 32, ks, lane);
+        if (F_KS || R_KS) lds_fence_all(f, r);
 #pragma unroll
-            for (int i = 0; i < 2; ++i) acc[j][i] = Mfma<TC>::run(f[j], r[i], acc[j][i]);
+        for (int j = 0; j < C::FB; ++j)
+#pragma unroll
+            for (int i = 0; i < C::RB; ++i) acc[j][i] = Mfma<TC>::run(f[j], r[i], acc[j][i]);
     }
 }
 
@@ -172,7 +224,6 @@ template <typename TC> __device__ __forceinline__ float from_bits16(unsigned sho
     c.u = u;
     return (float)c.t;
 }
-
 template <typename TC> __device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
     uint2 o;
     o.x = bits16<TC>(a) | ((unsigned)bits16<TC>(b) << 16);
@@ -205,10 +256,11 @@ struct EsmmK {
     void* ws;   // slots > 0 write here ([slot-1][T][N]) when set: the slots are summed afterwards
 };
 
-template <typename TC, bool W_IN_OUT, bool OUT32>
-__global__ __launch_bounds__(NT, 2) void esmm16_dma_kernel(EsmmK p) {
+template <typename TC, bool W_IN_OUT, bool OUT32, typename C>
+__global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
+    constexpr int BM = C::BM, BN = C::BN, STAGES = C::STAGES, NW = C::NW;
     extern __shared__ __attribute__((aligned(1024))) char smem[];
-    int* sTok = reinterpret_cast<int*>(smem + STAGES * STAGE_BYTES);
+    int* sTok = reinterpret_cast<int*>(smem + C::STAGE_AREA);
 
     const long logical = logical_tile(p.group);
     if (logical >= p.total) return;
@@ -222,154 +274,165 @@ __global__ __launch_bounds__(NT, 2) void esmm16_dma_kernel(EsmmK p) {
     const int n0 = nt * BN;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wr = wave >> 1, wf = wave & 1;
+    const int wr = wave / C::WF, wf = wave % C::WF;
     const int K = p.K, N = p.N;
 
     if (tid < BM) sTok[tid] = tid < rows ? p.token_ids[(size_t)s * p.T + row_start + tid] : -1;
     __syncthreads();
 
-    // ---- source pointers of this lane's copies (two wavefront copies per operand per stage) ----
+    // ---- source pointers of this lane's copies ----
     const char* zero = reinterpret_cast<const char*>(g_zero_block);
-    const char* srcA[2]; int stepA[2];
-    const char* srcB[2]; int stepB[2];
+    const char* srcR[C::R_CPW]; int stepR[C::R_CPW];
+    const char* srcF[C::F_CPW]; int stepF[C::F_CPW];
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-        {   // token rows, KC: chunk (wave + 4c) covers rows 16*chunk .. +15
-            const int row = 16 * (wave + 4 * c) + (lane >> 2);
-            const int kc = (lane & 3) ^ ((row >> 2) & 3);
-            const int tok = sTok[row];
-            const bool ok = tok >= 0;
-            srcA[c] = ok ? reinterpret_cast<const char*>(p.x) + (((size_t)p.x_slot_rows * s + tok) * K + kc * 8) * 2 : zero;
-            stepA[c] = ok ? BK * 2 : 0;
-        }
-        if (W_IN_OUT) {  // w[e][k][n], KS: chunk covers k rows 4*chunk .. +3, 16 pieces of 8 columns
-            const int kk = 4 * (wave + 4 * c) + (lane >> 4);
-            const int ch = (lane & 15) ^ ((kk & 3) << 2);
+    for (int i = 0; i < C::R_CPW; ++i) {   // token rows, KC
+        int row, kc;
+        kc_lane(wave + NW * i, lane, row, kc);
+        const int tok = sTok[row];
+        const bool ok = tok >= 0;
+        srcR[i] = ok ? reinterpret_cast<const char*>(p.x) + (((size_t)p.x_slot_rows * s + tok) * K + kc * 8) * 2 : zero;
+        stepR[i] = ok ? BK * 2 : 0;
+    }
+#pragma unroll
+    for (int i = 0; i < C::F_CPW; ++i) {
+        if (W_IN_OUT) {  // w[e][k][n], KS
+            int kk, ch;
+            ks_lane<BN>(wave + NW * i, lane, kk, ch);
             const int n = n0 + ch * 8;
             const bool ok = n < N;
-            srcB[c] = ok ? reinterpret_cast<const char*>(p.w) + (((size_t)e * K + kk) * N + n) * 2 : zero;
-            stepB[c] = ok ? BK * N * 2 : 0;
+            srcF[i] = ok ? reinterpret_cast<const char*>(p.w) + (((size_t)e * K + kk) * N + n) * 2 : zero;
+            stepF[i] = ok ? BK * N * 2 : 0;
         } else {         // w[e][n][k], KC
-            const int row = 16 * (wave + 4 * c) + (lane >> 2);
-            const int kc = (lane & 3) ^ ((row >> 2) & 3);
+            int row, kc;
+            kc_lane(wave + NW * i, lane, row, kc);
             const int n = n0 + row;
             const bool ok = n < N;
-            srcB[c] = ok ? reinterpret_cast<const char*>(p.w) + (((size_t)e * N + n) * K + kc * 8) * 2 : zero;
-            stepB[c] = ok ? BK * 2 : 0;
+            srcF[i] = ok ? reinterpret_cast<const char*>(p.w) + (((size_t)e * N + n) * K + kc * 8) * 2 : zero;
+            stepF[i] = ok ? BK * 2 : 0;
         }
     }
-    auto issue = [&](int stage) {   // 4 copies per lane
-        char* base = smem + stage * STAGE_BYTES;
+    auto issue = [&](int stage) {
+        char* base = smem + stage * C::STAGE_BYTES;
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            dma16(srcA[c], base + (wave + 4 * c) * 1024);
-            dma16(srcB[c], base + TILE_BYTES + (wave + 4 * c) * 1024);
-            srcA[c] += stepA[c];
-            srcB[c] += stepB[c];
+        for (int i = 0; i < C::R_CPW; ++i) {
+            dma16(srcR[i], base + (wave + NW * i) * 1024);
+            srcR[i] += stepR[i];
+        }
+#pragma unroll
+        for (int i = 0; i < C::F_CPW; ++i) {
+            dma16(srcF[i], base + C::R_BYTES + (wave + NW * i) * 1024);
+            srcF[i] += stepF[i];
         }
     };
 
-    f32x16 acc[2][2];
+    f32x16 acc[C::FB][C::RB];
     zero_acc(acc);
     const int nk = K / BK;
-    // prologue: STAGES-1 steps in flight (empty groups keep the wait counts uniform)
 #pragma unroll
     for (int st = 0; st < STAGES - 1; ++st)
         if (st < nk) issue(st);
     for (int kt = 0; kt < nk; ++kt) {
         // copies of step kt have landed when at most the copies of the later steps are outstanding
-        const int ahead = min(nk - 1 - kt, STAGES - 2);
-        if (ahead >= 2) wait_vmcnt<8>();
-        else if (ahead == 1) wait_vmcnt<4>();
-        else wait_vmcnt<0>();
+        wait_groups<C::CPW, STAGES - 2>(min(nk - 1 - kt, STAGES - 2));
         barrier_nofence();  // everyone's copies of step kt are in LDS; everyone is done reading step kt-1
         if (kt + STAGES - 1 < nk) issue((kt + STAGES - 1) % STAGES);
-        const char* base = smem + (kt % STAGES) * STAGE_BYTES;
-        mma_stage<TC, W_IN_OUT, false>(base, base + TILE_BYTES, wr, wf, lane, acc);
+        const char* base = smem + (kt % STAGES) * C::STAGE_BYTES;
+        mma_stage<TC, C, W_IN_OUT, false>(base, base + C::R_BYTES, wr, wf, lane, acc);
     }
 
     // ---- epilogue: lane holds, per 32x32 block, token row l%32 and 4 consecutive columns per group ----
+    // 16-bit results leave through LDS (PR rows per pass) so that BN/8 lanes write one contiguous row
+    // piece; fp32 results are stored from the registers, 16 bytes per lane.
     const bool to_ws = p.ws != nullptr && s > 0;
     void* const outp = to_ws ? p.ws : p.out;
     const bool accumulate = p.accumulate != 0 && !to_ws;
     const bool gelu = p.act == HEXA_ACT_GELU;
     const size_t out_base = to_ws ? (size_t)p.T * (s - 1) : (size_t)p.out_slot_rows * s;
     constexpr int CP = BN * 2 + 16;  // pitch (bytes) of the staged 16-bit result tile
-    if (!OUT32) barrier_nofence();   // the stage buffers are reused for the result tile
+    constexpr int PR = (BM * CP <= C::STAGE_AREA) ? BM : ((BM / 2) * CP <= C::STAGE_AREA ? BM / 2 : BM / 4);
+    static_assert(PR * CP <= C::STAGE_AREA, "the staged result must fit in the stage buffers");
+    constexpr int NPASS = OUT32 ? 1 : BM / PR;
+    constexpr int RW = 32 * C::RB, FW = 32 * C::FB;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int pass = 0; pass < NPASS; ++pass) {
+        if (!OUT32) { if (pass == 0) barrier_nofence(); else __syncthreads(); }   // staging area is free
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int nl = wf * 64 + j * 32 + 8 * g + 4 * (lane >> 5);
-            const int n = n0 + nl;
-            float bv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (p.bias && n < N) {
-                if (p.bias_dt == HEXA_F32) {
-                    const float4 b4 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.bias) + (size_t)e * N + n);
-                    bv[0] = b4.x; bv[1] = b4.y; bv[2] = b4.z; bv[3] = b4.w;
-                } else {
-                    const uint2 b2 = *reinterpret_cast<const uint2*>(reinterpret_cast<const unsigned short*>(p.bias) + (size_t)e * N + n);
-                    bv[0] = from_bits16<TC>(b2.x & 0xffff); bv[1] = from_bits16<TC>(b2.x >> 16);
-                    bv[2] = from_bits16<TC>(b2.y & 0xffff); bv[3] = from_bits16<TC>(b2.y >> 16);
+        for (int j = 0; j < C::FB; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int nl = wf * FW + j * 32 + 8 * g + 4 * (lane >> 5);
+                const int n = n0 + nl;
+                float bv[4] = {0.f, 0.f, 0.f, 0.f};
+                if (p.bias && n < N) {
+                    if (p.bias_dt == HEXA_F32) {
+                        const float4 b4 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.bias) + (size_t)e * N + n);
+                        bv[0] = b4.x; bv[1] = b4.y; bv[2] = b4.z; bv[3] = b4.w;
+                    } else {
+                        const uint2 b2 = *reinterpret_cast<const uint2*>(reinterpret_cast<const unsigned short*>(p.bias) + (size_t)e * N + n);
+                        bv[0] = from_bits16<TC>(b2.x & 0xffff); bv[1] = from_bits16<TC>(b2.x >> 16);
+                        bv[2] = from_bits16<TC>(b2.y & 0xffff); bv[3] = from_bits16<TC>(b2.y >> 16);
+                    }
                 }
-            }
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int rl = wr * 64 + i * 32 + (lane & 31);
-                float v[4];
+                for (int i = 0; i < C::RB; ++i) {
+                    const int rl = wr * RW + i * 32 + (lane & 31);
+                    if (!OUT32 && (wr * RW + i * 32) / PR != pass) continue;
+                    float v[4];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) v[q] = acc[j][i][4 * g + q] + bv[q];
-                if (OUT32) {
-                    const int tok = sTok[rl];
-                    if (tok < 0 || n >= N) continue;
-                    const size_t off = (out_base + tok) * N + n;
-                    float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(outp) + off);
-                    if (accumulate) { const float4 old = *dst; v[0] += old.x; v[1] += old.y; v[2] += old.z; v[3] += old.w; }
-                    *dst = make_float4(v[0], v[1], v[2], v[3]);
-                    if (gelu)
-                        *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.out_act) + off) =
-                            make_float4(gelu_fast(v[0]), gelu_fast(v[1]), gelu_fast(v[2]), gelu_fast(v[3]));
-                } else {
-                    *reinterpret_cast<uint2*>(smem + rl * CP + nl * 2) = pack4<TC>(v[0], v[1], v[2], v[3]);
+                    for (int q = 0; q < 4; ++q) v[q] = acc[j][i][4 * g + q] + bv[q];
+                    if (OUT32) {
+                        const int tok = sTok[rl];
+                        if (tok < 0 || n >= N) continue;
+                        const size_t off = (out_base + tok) * N + n;
+                        float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(outp) + off);
+                        if (accumulate) { const float4 old = *dst; v[0] += old.x; v[1] += old.y; v[2] += old.z; v[3] += old.w; }
+                        *dst = make_float4(v[0], v[1], v[2], v[3]);
+                        if (gelu)
+                            *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.out_act) + off) =
+                                make_float4(gelu_fast(v[0]), gelu_fast(v[1]), gelu_fast(v[2]), gelu_fast(v[3]));
+                    } else {
+                        *reinterpret_cast<uint2*>(smem + (rl - pass * PR) * CP + nl * 2) = pack4<TC>(v[0], v[1], v[2], v[3]);
+                    }
                 }
             }
         }
-    }
-    if (!OUT32) {
-        // 16-bit results leave through LDS so that 16 lanes write one contiguous 256-byte row piece
-        __syncthreads();
-        const int c = tid & 15, n = n0 + c * 8;
-        if (n < N) {
+        if (!OUT32) {
+            __syncthreads();
+            constexpr int LPR = BN / 8;             // lanes per row
+            constexpr int RPI = C::NT / LPR;        // rows per iteration
+            const int c = tid % LPR, n = n0 + c * 8;
+            if (n < N) {
+#pragma unroll 4
+                for (int it = 0; it < PR / RPI; ++it) {
+                    const int rl = it * RPI + tid / LPR;
+                    const int tok = sTok[pass * PR + rl];
+                    if (tok < 0) continue;
+                    const size_t off = (out_base + tok) * N + n;
+                    uint4 val = *reinterpret_cast<const uint4*>(smem + rl * CP + c * 16);
+                    uint4* dst = reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(outp) + off);
+                    if (accumulate) {
+                        const uint4 old = *dst;
+                        const unsigned ow[4] = {old.x, old.y, old.z, old.w};
+                        unsigned vw[4] = {val.x, val.y, val.z, val.w};
 #pragma unroll
-            for (int it = 0; it < BM / 16; ++it) {
-                const int rl = it * 16 + (tid >> 4);
-                const int tok = sTok[rl];
-                if (tok < 0) continue;
-                const size_t off = (out_base + tok) * N + n;
-                uint4 val = *reinterpret_cast<const uint4*>(smem + rl * CP + c * 16);
-                uint4* dst = reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(outp) + off);
-                if (accumulate) {
-                    const uint4 old = *dst;
-                    const unsigned ow[4] = {old.x, old.y, old.z, old.w};
-                    unsigned vw[4] = {val.x, val.y, val.z, val.w};
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const float lo = from_bits16<TC>(vw[q] & 0xffff) + from_bits16<TC>(ow[q] & 0xffff);
-                        const float hi = from_bits16<TC>(vw[q] >> 16) + from_bits16<TC>(ow[q] >> 16);
-                        vw[q] = bits16<TC>(lo) | ((unsigned)bits16<TC>(hi) << 16);
+                        for (int q = 0; q < 4; ++q) {
+                            const float lo = from_bits16<TC>(vw[q] & 0xffff) + from_bits16<TC>(ow[q] & 0xffff);
+                            const float hi = from_bits16<TC>(vw[q] >> 16) + from_bits16<TC>(ow[q] >> 16);
+                            vw[q] = bits16<TC>(lo) | ((unsigned)bits16<TC>(hi) << 16);
+                        }
+                        val = make_uint4(vw[0], vw[1], vw[2], vw[3]);
                     }
-                    val = make_uint4(vw[0], vw[1], vw[2], vw[3]);
-                }
-                *dst = val;
-                if (gelu) {
-                    // applied to the value as stored (rounded), like act(y1) on the tensor
-                    unsigned vw[4] = {val.x, val.y, val.z, val.w};
+                    *dst = val;
+                    if (gelu) {
+                        // applied to the value as stored (rounded), like act(y1) on the tensor
+                        unsigned vw[4] = {val.x, val.y, val.z, val.w};
 #pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        vw[q] = bits16<TC>(gelu_fast(from_bits16<TC>(vw[q] & 0xffff))) |
-                                ((unsigned)bits16<TC>(gelu_fast(from_bits16<TC>(vw[q] >> 16))) << 16);
-                    *reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(p.out_act) + off) =
-                        make_uint4(vw[0], vw[1], vw[2], vw[3]);
+                        for (int q = 0; q < 4; ++q)
+                            vw[q] = bits16<TC>(gelu_fast(from_bits16<TC>(vw[q] & 0xffff))) |
+                                    ((unsigned)bits16<TC>(gelu_fast(from_bits16<TC>(vw[q] >> 16))) << 16);
+                        *reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(p.out_act) + off) =
+                            make_uint4(vw[0], vw[1], vw[2], vw[3]);
+                    }
                 }
             }
         }
@@ -389,13 +452,20 @@ template <typename K> int ensure_smem(K kernel, int bytes) {
     return HEXA_OK;
 }
 
-template <typename TC, bool IO, bool OUT32>
+template <typename TC, bool IO, bool OUT32, typename C>
 int launch_esmm_dma_t(EsmmK& p, int grid, hipStream_t st) {
-    auto kernel = esmm16_dma_kernel<TC, IO, OUT32>;
-    if (int rc = ensure_smem(kernel, SMEM_BYTES)) return rc;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), SMEM_BYTES, st, p);
+    auto kernel = esmm16_dma_kernel<TC, IO, OUT32, C>;
+    constexpr int bytes = C::STAGE_AREA + C::BM * 4;
+    if (int rc = ensure_smem(kernel, bytes)) return rc;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(C::NT), bytes, st, p);
     HEXA_CHECK_LAUNCH("esmm16_dma");
     return HEXA_OK;
+}
+
+template <typename TC, typename C>
+int launch_esmm_dma_d(EsmmK& p, int grid, bool io, bool o32, hipStream_t st) {
+    if (o32) return io ? launch_esmm_dma_t<TC, true, true, C>(p, grid, st) : launch_esmm_dma_t<TC, false, true, C>(p, grid, st);
+    return io ? launch_esmm_dma_t<TC, true, false, C>(p, grid, st) : launch_esmm_dma_t<TC, false, false, C>(p, grid, st);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -403,9 +473,6 @@ int launch_esmm_dma_t(EsmmK& p, int grid, hipStream_t st) {
 // ------------------------------------------------------------------------------------------------
 constexpr int MAX_SLOTS = 8;      // routing slots handled by this path
 constexpr int TOK_RING = 8;       // steps of token ids kept in LDS (32 ids each)
-constexpr int ESTMM_STAGE_AREA = 128 * (BN + 4) * 4;   // >= STAGES * STAGE_BYTES: also holds the staged fp32 result
-constexpr int ESTMM_SMEM_BYTES = ESTMM_STAGE_AREA + TOK_RING * 32 * 4;
-static_assert(ESTMM_STAGE_AREA >= STAGES * STAGE_BYTES, "result staging must cover the stage buffers");
 
 struct EstmmK {
     const void* pm; const void* qm; void* dw;
@@ -420,13 +487,21 @@ struct Cursor {   // walks the expert's token list in 32-token steps, slot after
     int s, r;
 };
 
-template <typename TC, bool OUT32>
-__global__ __launch_bounds__(NT, 2) void estmm16_dma_kernel(EstmmK p) {
-    extern __shared__ __attribute__((aligned(1024))) char smem[];
-    int* sIds = reinterpret_cast<int*>(smem + ESTMM_STAGE_AREA);       // [TOK_RING][32]
-    __shared__ int sBeg[MAX_SLOTS], sEnd[MAX_SLOTS];
+// fp32 result rows staged per pass, and the LDS area that holds both the stages and that staging
+template <typename C> constexpr int estmm_pass_rows() { return C::BN <= 128 ? 128 : 64; }
+template <typename C> constexpr int estmm_stage_area() {
+    constexpr int staged = estmm_pass_rows<C>() * (C::BN + 4) * 4;
+    return C::STAGE_AREA > staged ? C::STAGE_AREA : staged;
+}
 
+template <typename TC, bool OUT32, typename C>
+__global__ __launch_bounds__(C::NT, C::MINW) void estmm16_dma_kernel(EstmmK p) {
+    constexpr int BM = C::BM, BN = C::BN, STAGES = C::STAGES, NW = C::NW;
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    int* sIds = reinterpret_cast<int*>(smem + estmm_stage_area<C>());       // [TOK_RING][32]
+    __shared__ int sBeg[MAX_SLOTS], sEnd[MAX_SLOTS];
     __shared__ int sExpert;
+
     const long logical = logical_tile(p.group);
     if (logical >= p.total) return;
     const int per_e = p.mtn * p.ntn;
@@ -435,25 +510,27 @@ __global__ __launch_bounds__(NT, 2) void estmm16_dma_kernel(EstmmK p) {
     const int m0 = (rem / p.ntn) * BM, n0 = (rem % p.ntn) * BN;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wr = wave >> 1, wf = wave & 1;
+    const int wr = wave / C::WF, wf = wave % C::WF;
     const int M = p.M, N = p.N, T = p.T, nslot = p.k;
 
     // Heaviest experts first: workgroups are dispatched in id order, so giving the long token lists
     // to the first ones shortens the tail.  The expert of this workgroup is the one whose load has
     // rank `rank` (ties broken by index).  Up to 256 experts; beyond that the order is by index.
     int e = rank;
-    if (p.E <= NT) {
-        auto load_of = [&](int x) {
+    if (p.E <= 256) {
+        __shared__ int sLoad[256];
+        if (tid < p.E) {
             int t = 0;
             for (int s = 0; s < nslot; ++s)
-                t += p.offsets[(size_t)s * (p.E + 1) + x + 1] - p.offsets[(size_t)s * (p.E + 1) + x];
-            return t;
-        };
+                t += p.offsets[(size_t)s * (p.E + 1) + tid + 1] - p.offsets[(size_t)s * (p.E + 1) + tid];
+            sLoad[tid] = t;
+        }
+        __syncthreads();
         if (tid < p.E) {
-            const int mine = load_of(tid);
+            const int mine = sLoad[tid];
             int r = 0;
             for (int x = 0; x < p.E; ++x) {
-                const int o = load_of(x);
+                const int o = sLoad[x];
                 r += (o > mine || (o == mine && x < tid)) ? 1 : 0;
             }
             if (r == rank) sExpert = tid;
@@ -491,33 +568,45 @@ __global__ __launch_bounds__(NT, 2) void estmm16_dma_kernel(EstmmK p) {
             __builtin_amdgcn_global_load_lds((glb_ptr_t)src, (lds_ptr_t)(sIds + (step % TOK_RING) * 32), 4, 0, 0);
     };
     // operand tiles of one step (token ids of the step are already in LDS)
-    const int ch0 = lane & 15;
     auto issue_data = [&](int step, Cursor c) {
-        char* base = smem + (step % STAGES) * STAGE_BYTES;
+        char* base = smem + (step % STAGES) * C::STAGE_BYTES;
         const unsigned ids = lds_addr(sIds + (step % TOK_RING) * 32);
         const int end = sEnd[c.s];
-        int toks[2];
+        int kkR[C::R_CPW], chR[C::R_CPW], kkF[C::F_CPW], chF[C::F_CPW];
+        int tokR[C::R_CPW], tokF[C::F_CPW];
 #pragma unroll
-        for (int cc = 0; cc < 2; ++cc) toks[cc] = lds_read_i32(ids + 4 * (4 * (wave + 4 * cc) + (lane >> 4)));
-        lds_fence(toks[0], toks[1]);
+        for (int i = 0; i < C::R_CPW; ++i) {
+            ks_lane<BM>(wave + NW * i, lane, kkR[i], chR[i]);
+            tokR[i] = lds_read_i32(ids + 4 * kkR[i]);
+        }
 #pragma unroll
-        for (int cc = 0; cc < 2; ++cc) {
-            const int kk = 4 * (wave + 4 * cc) + (lane >> 4);
-            const int ch = ch0 ^ ((kk & 3) << 2);
-            const bool row_ok = c.r + kk < end;
-            const int tok = toks[cc];
-            const bool okp = row_ok && (m0 + ch * 8 < M), okq = row_ok && (n0 + ch * 8 < N);
-            const char* sp = okp ? reinterpret_cast<const char*>(p.pm) + (((size_t)p.p_slot_rows * c.s + tok) * M + m0 + ch * 8) * 2 : zero;
-            const char* sq = okq ? reinterpret_cast<const char*>(p.qm) + (((size_t)p.q_slot_rows * c.s + tok) * N + n0 + ch * 8) * 2 : zero;
-            dma16(sp, base + (wave + 4 * cc) * 1024);
-            dma16(sq, base + TILE_BYTES + (wave + 4 * cc) * 1024);
+        for (int i = 0; i < C::F_CPW; ++i) {
+            ks_lane<BN>(wave + NW * i, lane, kkF[i], chF[i]);
+            tokF[i] = lds_read_i32(ids + 4 * kkF[i]);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < C::R_CPW; ++i) {
+            int tok = tokR[i];
+            asm volatile("" : "+v"(tok));   // consumed only after the wait above
+            const bool ok = (c.r + kkR[i] < end) && (m0 + chR[i] * 8 < M);
+            const char* sp = ok ? reinterpret_cast<const char*>(p.pm) + (((size_t)p.p_slot_rows * c.s + tok) * M + m0 + chR[i] * 8) * 2 : zero;
+            dma16(sp, base + (wave + NW * i) * 1024);
+        }
+#pragma unroll
+        for (int i = 0; i < C::F_CPW; ++i) {
+            int tok = tokF[i];
+            asm volatile("" : "+v"(tok));
+            const bool ok = (c.r + kkF[i] < end) && (n0 + chF[i] * 8 < N);
+            const char* sq = ok ? reinterpret_cast<const char*>(p.qm) + (((size_t)p.q_slot_rows * c.s + tok) * N + n0 + chF[i] * 8) * 2 : zero;
+            dma16(sq, base + C::R_BYTES + (wave + NW * i) * 1024);
         }
     };
 
-    f32x16 acc[2][2];
+    f32x16 acc[C::FB][C::RB];
     zero_acc(acc);
     if (nsteps > 0) {
-        // Copy groups of 5 per wavefront: { data(step x) [4 copies], ids(step x + LEAD) [1 copy] }.
+        // Copy groups of CPW+1 per wavefront: { data(step x) [CPW copies], ids(step x + LEAD) [1 copy] }.
         // Group x is issued LEAD steps before step x is consumed, so when group kt has landed the ids
         // needed to issue data(kt + LEAD) are in LDS as well.
         constexpr int LEAD = STAGES - 1;
@@ -533,51 +622,55 @@ __global__ __launch_bounds__(NT, 2) void estmm16_dma_kernel(EstmmK p) {
             }
         }
         for (int kt = 0; kt < nsteps; ++kt) {
-            const int ahead = min(nsteps - 1 - kt, LEAD - 1);   // groups issued after group kt
-            if (ahead >= 2) wait_vmcnt<10>();
-            else if (ahead == 1) wait_vmcnt<5>();
-            else wait_vmcnt<0>();
+            wait_groups<C::CPW + 1, LEAD - 1>(min(nsteps - 1 - kt, LEAD - 1));   // groups issued after group kt
             barrier_nofence();
             const int jd = kt + LEAD;
             if (jd < nsteps) {
                 issue_data(jd, cdat); cdat = advance(cdat);
                 issue_ids(jd + LEAD, cid); cid = advance(cid);
             }
-            const char* base = smem + (kt % STAGES) * STAGE_BYTES;
-            mma_stage<TC, true, true>(base, base + TILE_BYTES, wr, wf, lane, acc);
+            const char* base = smem + (kt % STAGES) * C::STAGE_BYTES;
+            mma_stage<TC, C, true, true>(base, base + C::R_BYTES, wr, wf, lane, acc);
         }
     } else if (p.accumulate) {
         return;
     }
 
     // ---- epilogue: lane holds row m = l%32 of a block and 4 consecutive n per group ----
-    // The block leaves through LDS (pitch 132 floats) so that 32 lanes write one contiguous 512-byte
-    // row of dw; 16-bit results are packed on the way out.
+    // The block leaves through LDS, PRF rows at a time (pitch BN+4 floats), so that BN/4 lanes write
+    // one contiguous row of dw; 16-bit results are packed on the way out.
     const bool accumulate = p.accumulate != 0;
-    constexpr int CPF = BN + 4;   // floats per staged row
     float* sC = reinterpret_cast<float*>(smem);
-    barrier_nofence();            // all wavefronts are done reading the stage buffers
+    constexpr int CPF = BN + 4;
+    constexpr int PRF = estmm_pass_rows<C>();
+    constexpr int LPRF = BN / 4;              // lanes per row
+    constexpr int RPI = C::NT / LPRF;         // rows stored per iteration
+    constexpr int RW = 32 * C::RB, FW = 32 * C::FB;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int ml = wr * 64 + i * 32 + (lane & 31);
+    for (int h = 0; h < BM / PRF; ++h) {
+        if (h == 0) barrier_nofence(); else __syncthreads();   // stage buffers / previous pass are free
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int i = 0; i < C::RB; ++i) {
+            const int mb = wr * RW + i * 32;          // first row of this 32-row block inside the tile
+            if (mb / PRF != h) continue;
+            const int ml = mb - h * PRF + (lane & 31);
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int nl = wf * 64 + j * 32 + 8 * g + 4 * (lane >> 5);
-                *reinterpret_cast<float4*>(sC + ml * CPF + nl) =
-                    make_float4(acc[j][i][4 * g], acc[j][i][4 * g + 1], acc[j][i][4 * g + 2], acc[j][i][4 * g + 3]);
+            for (int j = 0; j < C::FB; ++j) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int nl = wf * FW + j * 32 + 8 * g + 4 * (lane >> 5);
+                    *reinterpret_cast<float4*>(sC + ml * CPF + nl) =
+                        make_float4(acc[j][i][4 * g], acc[j][i][4 * g + 1], acc[j][i][4 * g + 2], acc[j][i][4 * g + 3]);
+                }
             }
         }
-    }
-    __syncthreads();
-    {
-        const int c = tid & 31, n = n0 + c * 4;
+        __syncthreads();
+        const int c = tid % LPRF, n = n0 + c * 4;
         if (n < N) {
 #pragma unroll 4
-            for (int it = 0; it < BM / 8; ++it) {
-                const int ml = it * 8 + (tid >> 5);
-                const int m = m0 + ml;
+            for (int it = 0; it < PRF / RPI; ++it) {
+                const int ml = it * RPI + tid / LPRF;
+                const int m = m0 + h * PRF + ml;
                 if (m >= M) break;
                 float4 v = *reinterpret_cast<const float4*>(sC + ml * CPF + c * 4);
                 const size_t off = ((size_t)e * M + m) * N + n;
@@ -599,33 +692,23 @@ __global__ __launch_bounds__(NT, 2) void estmm16_dma_kernel(EstmmK p) {
     }
 }
 
-
-template <typename TC, bool OUT32>
+template <typename TC, bool OUT32, typename C>
 int launch_estmm_dma_t(EstmmK& p, int grid, hipStream_t st) {
-    auto kernel = estmm16_dma_kernel<TC, OUT32>;
-    if (int rc = ensure_smem(kernel, ESTMM_SMEM_BYTES)) return rc;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), ESTMM_SMEM_BYTES, st, p);
+    auto kernel = estmm16_dma_kernel<TC, OUT32, C>;
+    constexpr int bytes = estmm_stage_area<C>() + TOK_RING * 32 * 4;
+    if (int rc = ensure_smem(kernel, bytes)) return rc;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(C::NT), bytes, st, p);
     HEXA_CHECK_LAUNCH("estmm16_dma");
     return HEXA_OK;
 }
 
-}  // namespace
-
-bool esmm16_dma_supported(const EsmmArgs& a) {
-    return a.w_dt == a.x_dt && (a.in_dim % BK) == 0 && (a.out_dim % 8) == 0 &&
-           (a.out_dt == a.x_dt || a.out_dt == HEXA_F32);
-}
-
-bool estmm16_dma_supported(const EstmmArgs& a) {
-    return a.r.k <= MAX_SLOTS && (a.m_dim % 8) == 0 && (a.n_dim % 8) == 0 && (a.dw_dt == a.pq_dt || a.dw_dt == HEXA_F32);
-}
-
-int launch_estmm16_dma(const EstmmArgs& a, hipStream_t st) {
+template <typename C>
+int launch_estmm_dma_c(const EstmmArgs& a, hipStream_t st) {
     EstmmK p;
     p.pm = a.p; p.qm = a.q; p.dw = a.dw;
     p.token_ids = a.r.token_ids; p.offsets = a.r.offsets;
     p.T = a.r.T; p.k = a.r.k; p.E = a.r.E; p.M = a.m_dim; p.N = a.n_dim;
-    p.mtn = div_up(a.m_dim, BM); p.ntn = div_up(a.n_dim, BN);
+    p.mtn = div_up(a.m_dim, C::BM); p.ntn = div_up(a.n_dim, C::BN);
     p.p_slot_rows = a.p_per_slot ? a.r.T : 0;
     p.q_slot_rows = a.q_per_slot ? a.r.T : 0;
     p.accumulate = a.accumulate;
@@ -634,20 +717,24 @@ int launch_estmm16_dma(const EstmmArgs& a, hipStream_t st) {
     if (p.total == 0) return HEXA_OK;
     const int grid = round_up(p.total, 8 * p.group);
     const bool o32 = a.dw_dt == HEXA_F32;
-    if (a.pq_dt == HEXA_BF16) return o32 ? launch_estmm_dma_t<__bf16, true>(p, grid, st) : launch_estmm_dma_t<__bf16, false>(p, grid, st);
-    return o32 ? launch_estmm_dma_t<_Float16, true>(p, grid, st) : launch_estmm_dma_t<_Float16, false>(p, grid, st);
+    if (a.pq_dt == HEXA_BF16) return o32 ? launch_estmm_dma_t<__bf16, true, C>(p, grid, st) : launch_estmm_dma_t<__bf16, false, C>(p, grid, st);
+    return o32 ? launch_estmm_dma_t<_Float16, true, C>(p, grid, st) : launch_estmm_dma_t<_Float16, false, C>(p, grid, st);
 }
 
-int launch_esmm16_dma(const EsmmArgs& a, hipStream_t st) {
+template <typename C>
+int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
     EsmmK p;
     p.x = a.x; p.w = a.w; p.bias = a.bias; p.out = a.out; p.out_act = a.out_act;
-    p.token_ids = a.r.token_ids; p.tile_info = a.r.tile_info; p.tile_count = a.r.tile_count;
-    p.T = a.r.T; p.K = a.in_dim; p.N = a.out_dim; p.mt_ub = a.r.mt_ub;
-    p.ntn = div_up(a.out_dim, BN);
+    p.token_ids = a.r.token_ids;
+    p.tile_info = large ? a.r.tile_info_l : a.r.tile_info;
+    p.tile_count = large ? a.r.tile_count_l : a.r.tile_count;
+    p.mt_ub = large ? a.r.mt_ub_l : a.r.mt_ub;
+    p.T = a.r.T; p.K = a.in_dim; p.N = a.out_dim;
+    p.ntn = div_up(a.out_dim, C::BN);
     p.x_slot_rows = a.x_per_slot ? a.r.T : 0;
     p.out_slot_rows = a.out_per_slot ? a.r.T : 0;
     p.bias_dt = a.bias_dt; p.out_dt = a.out_dt; p.act = a.act;
-    p.group = p.ntn * 4;
+    p.group = p.ntn * (large ? 2 : 4);
     // Summing the slots into one result: with scratch, every slot runs in ONE launch (slot 0 into
     // `out`, the others into the scratch) and a reduction adds them in slot order; without it, one
     // launch per slot, each adding into `out`.
@@ -663,18 +750,58 @@ int launch_esmm16_dma(const EsmmArgs& a, hipStream_t st) {
         const int grid = round_up(p.total, 8 * p.group);
         const bool io = a.w_layout == HEXA_W_IN_OUT;
         const bool o32 = a.out_dt == HEXA_F32;
-        int rc;
-        if (a.x_dt == HEXA_BF16) {
-            if (o32) rc = io ? launch_esmm_dma_t<__bf16, true, true>(p, grid, st) : launch_esmm_dma_t<__bf16, false, true>(p, grid, st);
-            else rc = io ? launch_esmm_dma_t<__bf16, true, false>(p, grid, st) : launch_esmm_dma_t<__bf16, false, false>(p, grid, st);
-        } else {
-            if (o32) rc = io ? launch_esmm_dma_t<_Float16, true, true>(p, grid, st) : launch_esmm_dma_t<_Float16, false, true>(p, grid, st);
-            else rc = io ? launch_esmm_dma_t<_Float16, true, false>(p, grid, st) : launch_esmm_dma_t<_Float16, false, false>(p, grid, st);
-        }
+        const int rc = a.x_dt == HEXA_BF16 ? launch_esmm_dma_d<__bf16, C>(p, grid, io, o32, st)
+                                           : launch_esmm_dma_d<_Float16, C>(p, grid, io, o32, st);
         if (rc) return rc;
     }
     if (p.ws) return launch_sum_slots(a.out, a.slot_ws, (int64_t)a.r.T * a.out_dim, a.r.k - 1, a.out_dt, st);
     return HEXA_OK;
+}
+
+// 0: automatic; 1: 128x128; 2: 256x128 (8 wavefronts); 3: 256x128 (4 wavefronts); 4: 256x256
+// (HEXA_MOE_TILE, testing aid, read once)
+int forced_tile() {
+    static const int v = [] { const char* s = getenv("HEXA_MOE_TILE"); return s ? atoi(s) : 0; }();
+    return v;
+}
+
+int pick_esmm_tile(long rows, int cols) {
+    const int f = forced_tile();
+    if (f) return f;
+    return rows / 256 * div_up(cols, 128) >= 512 ? 2 : 1;
+}
+
+}  // namespace
+
+bool esmm16_dma_supported(const EsmmArgs& a) {
+    return a.w_dt == a.x_dt && (a.in_dim % BK) == 0 && (a.out_dim % 8) == 0 &&
+           (a.out_dt == a.x_dt || a.out_dt == HEXA_F32);
+}
+
+bool estmm16_dma_supported(const EstmmArgs& a) {
+    return a.r.k <= MAX_SLOTS && (a.m_dim % 8) == 0 && (a.n_dim % 8) == 0 && (a.dw_dt == a.pq_dt || a.dw_dt == HEXA_F32);
+}
+
+int launch_estmm16_dma(const EstmmArgs& a, hipStream_t st) {
+    switch (forced_tile()) {
+        case 2: return launch_estmm_dma_c<CfgL>(a, st);
+        case 3: return launch_estmm_dma_c<CfgM>(a, st);
+        case 4: return launch_estmm_dma_c<CfgX>(a, st);
+        case 5: return launch_estmm_dma_c<CfgX8>(a, st);
+        case 6: return launch_estmm_dma_c<CfgX16>(a, st);
+        default: return launch_estmm_dma_c<CfgS>(a, st);
+    }
+}
+
+int launch_esmm16_dma(const EsmmArgs& a, hipStream_t st) {
+    switch (pick_esmm_tile((long)a.r.T * a.r.k, a.out_dim)) {
+        case 2: return launch_esmm_dma_c<CfgL>(a, true, st);
+        case 3: return launch_esmm_dma_c<CfgM>(a, true, st);
+        case 4: return launch_esmm_dma_c<CfgX>(a, true, st);
+        case 5: return launch_esmm_dma_c<CfgX8>(a, true, st);
+        case 6: return launch_esmm_dma_c<CfgX16>(a, true, st);
+        default: return launch_esmm_dma_c<CfgS>(a, false, st);
+    }
 }
 
 }  // namespace hexa

@@ -39,7 +39,9 @@ struct RouteView {
     const int32_t* offsets;     // [k][E+1]
     const int4* tile_info;      // [k][mt_ub]: {expert, row_start, row_count, 0}
     const int32_t* tile_count;  // [k]
-    int T, k, E, mt_ub;
+    const int4* tile_info_l;    // the same with HEXA_TILE_ROWS_L rows per tile
+    const int32_t* tile_count_l;
+    int T, k, E, mt_ub, mt_ub_l;
 };
 
 RouteView route_view(const int32_t* route, int T, int k, int E);

@@ -60,48 +60,59 @@ __device__ __forceinline__ int block_excl_scan_256(int v, int* tmp, int& total) 
 // Given per-expert totals in LDS (tot[E]), write counts / offsets (exclusive prefix of the totals
 // rounded up to `pad`) and, when tile_info != nullptr, one record per kTileRows rows of each
 // segment.  LDS: tot[E], off[E+1], tbase[E+1], tmp[8].
-__device__ void finish_slot(const int32_t* tot, int32_t* off, int32_t* tbase, int* tmp, int E, int pad,
-                            int32_t* counts, int32_t* offsets, int4* tile_info, int32_t* tile_count,
-                            int mt_ub) {
+// One record per `rows_per_tile` rows of every expert segment (tbase: LDS scratch of E+1 ints).
+__device__ void emit_tiles(const int32_t* tot, const int32_t* off, int32_t* tbase, int* tmp, int E, int rows_per_tile,
+                           int4* tile_info, int32_t* tile_count, int mt_ub) {
     const int tid = threadIdx.x;
     const int chunk = (E + 255) / 256;
     const int e0 = min(E, tid * chunk), e1 = min(E, e0 + chunk);
-    int sum_rows = 0, sum_tiles = 0;
-    for (int e = e0; e < e1; ++e) {
-        int c = tot[e];
-        sum_rows += ((c + pad - 1) / pad) * pad;
-        sum_tiles += (c + kTileRows - 1) / kTileRows;
-    }
-    int total_rows, total_tiles;
-    int row_base = block_excl_scan_256(sum_rows, tmp, total_rows);
+    int sum_tiles = 0;
+    for (int e = e0; e < e1; ++e) sum_tiles += (tot[e] + rows_per_tile - 1) / rows_per_tile;
+    int total_tiles;
     int tile_base = block_excl_scan_256(sum_tiles, tmp, total_tiles);
     for (int e = e0; e < e1; ++e) {
-        int c = tot[e];
-        off[e] = row_base;
         tbase[e] = tile_base;
-        row_base += ((c + pad - 1) / pad) * pad;
-        tile_base += (c + kTileRows - 1) / kTileRows;
+        tile_base += (tot[e] + rows_per_tile - 1) / rows_per_tile;
     }
-    if (tid == 0) { off[E] = total_rows; tbase[E] = total_tiles; }
+    if (tid == 0) { tbase[E] = total_tiles; *tile_count = total_tiles; }
+    __syncthreads();
+    const int n = min(total_tiles, mt_ub);
+    for (int m = tid; m < n; m += 256) {
+        int lo = 0, hi = E;  // invariant: tbase[lo] <= m < tbase[hi]
+        while (hi - lo > 1) {
+            int mid = (lo + hi) >> 1;
+            if (tbase[mid] <= m) lo = mid; else hi = mid;
+        }
+        int j = m - tbase[lo];
+        int rows = min(rows_per_tile, tot[lo] - j * rows_per_tile);
+        tile_info[m] = make_int4(lo, off[lo] + j * rows_per_tile, rows, 0);
+    }
+    __syncthreads();
+}
+
+__device__ void finish_slot(const int32_t* tot, int32_t* off, int32_t* tbase, int* tmp, int E, int pad,
+                            int32_t* counts, int32_t* offsets, int4* tile_info, int32_t* tile_count,
+                            int mt_ub, int4* tile_info_l, int32_t* tile_count_l, int mt_ub_l) {
+    const int tid = threadIdx.x;
+    const int chunk = (E + 255) / 256;
+    const int e0 = min(E, tid * chunk), e1 = min(E, e0 + chunk);
+    int sum_rows = 0;
+    for (int e = e0; e < e1; ++e) sum_rows += ((tot[e] + pad - 1) / pad) * pad;
+    int total_rows;
+    int row_base = block_excl_scan_256(sum_rows, tmp, total_rows);
+    for (int e = e0; e < e1; ++e) {
+        off[e] = row_base;
+        row_base += ((tot[e] + pad - 1) / pad) * pad;
+    }
+    if (tid == 0) off[E] = total_rows;
     __syncthreads();
     for (int e = tid; e <= E; e += 256) {
         if (offsets) offsets[e] = off[e];
         if (counts && e < E) counts[e] = tot[e];
     }
     if (tile_info) {
-        if (tid == 0) *tile_count = total_tiles;
-        const int n = min(total_tiles, mt_ub);
-        for (int m = tid; m < n; m += 256) {
-            // last expert whose first tile index is <= m (experts without tiles share a base)
-            int lo = 0, hi = E;  // invariant: tbase[lo] <= m < tbase[hi]
-            while (hi - lo > 1) {
-                int mid = (lo + hi) >> 1;
-                if (tbase[mid] <= m) lo = mid; else hi = mid;
-            }
-            int j = m - tbase[lo];
-            int rows = min(kTileRows, tot[lo] - j * kTileRows);
-            tile_info[m] = make_int4(lo, off[lo] + j * kTileRows, rows, 0);
-        }
+        emit_tiles(tot, off, tbase, tmp, E, kTileRows, tile_info, tile_count, mt_ub);
+        emit_tiles(tot, off, tbase, tmp, E, HEXA_TILE_ROWS_L, tile_info_l, tile_count_l, mt_ub_l);
     }
 }
 
@@ -113,6 +124,8 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ u
                                                          int32_t* __restrict__ offsets,
                                                          int4* __restrict__ tile_info,
                                                          int32_t* __restrict__ tile_count, int mt_ub,
+                                                         int4* __restrict__ tile_info_l,
+                                                         int32_t* __restrict__ tile_count_l, int mt_ub_l,
                                                          int prefix_only) {
     extern __shared__ int32_t sh[];
     int32_t* tot = sh;
@@ -135,7 +148,8 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ u
     finish_slot(tot, off, tbase, tmp, E, pad, counts ? counts + (size_t)s * E : nullptr,
                 offsets ? offsets + (size_t)s * (E + 1) : nullptr,
                 tile_info ? tile_info + (size_t)s * mt_ub : nullptr, tile_count ? tile_count + s : nullptr,
-                mt_ub);
+                mt_ub, tile_info_l ? tile_info_l + (size_t)s * mt_ub_l : nullptr,
+                tile_count_l ? tile_count_l + s : nullptr, mt_ub_l);
 }
 
 template <typename IdxT>
@@ -188,7 +202,9 @@ __global__ __launch_bounds__(256) void route_from_lists_kernel(const int32_t* __
                                                                int T, int E, int32_t* __restrict__ counts,
                                                                int32_t* __restrict__ offsets,
                                                                int4* __restrict__ tile_info,
-                                                               int32_t* __restrict__ tile_count, int mt_ub) {
+                                                               int32_t* __restrict__ tile_count, int mt_ub,
+                                                               int4* __restrict__ tile_info_l,
+                                                               int32_t* __restrict__ tile_count_l, int mt_ub_l) {
     extern __shared__ int32_t sh[];
     int32_t* tot = sh;
     int32_t* off = tot + E;
@@ -206,7 +222,8 @@ __global__ __launch_bounds__(256) void route_from_lists_kernel(const int32_t* __
     }
     __syncthreads();
     finish_slot(tot, off, tbase, tmp, E, 1, counts + (size_t)s * E, offsets + (size_t)s * (E + 1),
-                tile_info + (size_t)s * mt_ub, tile_count + s, mt_ub);
+                tile_info + (size_t)s * mt_ub, tile_count + s, mt_ub, tile_info_l + (size_t)s * mt_ub_l,
+                tile_count_l + s, mt_ub_l);
 }
 
 int ceil_log2(int n) { int b = 0; while ((1 << b) < n) ++b; return b; }
@@ -223,6 +240,8 @@ extern "C" int hexa_route_layout_get(int T, int k, int E, hexa_route_layout* out
     if (T < 0 || k < 1 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_route_layout_get: bad sizes T=%d k=%d E=%d", T, k, E);
     const int64_t K = k;
     out->mt_ub = T / HEXA_TILE_ROWS + E;
+    out->mt_ub_l = T / HEXA_TILE_ROWS_L + E;
+    out->reserved = 0;
     out->units = T > 0 ? div_up(T, HEXA_ROUTE_UNIT) : 1;
     int64_t p = 0;
     out->counts = p;      p += K * E;
@@ -232,6 +251,9 @@ extern "C" int hexa_route_layout_get(int T, int k, int E, hexa_route_layout* out
     out->tile_count = p;  p += K;
     p = (p + 3) & ~(int64_t)3;  // tile records are 16-byte vectors
     out->tile_info = p;   p += K * out->mt_ub * 4;
+    out->tile_count_l = p; p += K;
+    p = (p + 3) & ~(int64_t)3;
+    out->tile_info_l = p; p += K * out->mt_ub_l * 4;
     out->scratch = p;     p += K * out->units * E;
     out->total_ints = p;
     return HEXA_OK;
@@ -246,7 +268,9 @@ RouteView route_view(const int32_t* route, int T, int k, int E) {
     v.offsets = route + L.offsets;
     v.tile_info = reinterpret_cast<const int4*>(route + L.tile_info);
     v.tile_count = route + L.tile_count;
-    v.T = T; v.k = k; v.E = E; v.mt_ub = L.mt_ub;
+    v.tile_info_l = reinterpret_cast<const int4*>(route + L.tile_info_l);
+    v.tile_count_l = route + L.tile_count_l;
+    v.T = T; v.k = k; v.E = E; v.mt_ub = L.mt_ub; v.mt_ub_l = L.mt_ub_l;
     return v;
 }
 }  // namespace hexa
@@ -276,7 +300,8 @@ extern "C" int hexa_route_build(const void* routing, int routing_is_i64, int64_t
     HEXA_CHECK_LAUNCH("route_hist");
     hipLaunchKernelGGL(route_scan_kernel, dim3(k), dim3(256), scan_lds_bytes(E), st, H, E, L.units, 1,
                        route + L.counts, route + L.offsets, reinterpret_cast<int4*>(route + L.tile_info),
-                       route + L.tile_count, L.mt_ub, 0);
+                       route + L.tile_count, L.mt_ub, reinterpret_cast<int4*>(route + L.tile_info_l),
+                       route + L.tile_count_l, L.mt_ub_l, 0);
     HEXA_CHECK_LAUNCH("route_scan");
     const int nbits = ceil_log2(E);
     if (routing_is_i64)
@@ -305,7 +330,8 @@ extern "C" int hexa_token_count(int32_t* tokens_per_expert, int32_t* expanded, c
                        (int64_t)1, (int64_t)0, T, E, units, scratch);
     HEXA_CHECK_LAUNCH("route_hist");
     hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(256), scan_lds_bytes(E), st, scratch, E, units, pad,
-                       tokens_per_expert, expanded, (int4*)nullptr, (int32_t*)nullptr, 0, 0);
+                       tokens_per_expert, expanded, (int4*)nullptr, (int32_t*)nullptr, 0, (int4*)nullptr,
+                       (int32_t*)nullptr, 0, 0);
     HEXA_CHECK_LAUNCH("route_scan");
     return HEXA_OK;
 }
@@ -321,7 +347,8 @@ extern "C" int hexa_token_assign(int32_t* token_idx_list, int32_t* expert_idx_li
                        (int64_t)1, (int64_t)0, T, E, units, scratch);
     HEXA_CHECK_LAUNCH("route_hist");
     hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(256), scan_lds_bytes(E), st, scratch, E, units, 1,
-                       (int32_t*)nullptr, (int32_t*)nullptr, (int4*)nullptr, (int32_t*)nullptr, 0, 1);
+                       (int32_t*)nullptr, (int32_t*)nullptr, (int4*)nullptr, (int32_t*)nullptr, 0, (int4*)nullptr,
+                       (int32_t*)nullptr, 0, 1);
     HEXA_CHECK_LAUNCH("route_scan");
     hipLaunchKernelGGL(route_scatter_kernel<int32_t>, dim3(units, 1), dim3(kWave), sizeof(int32_t) * E, st, routing,
                        (int64_t)1, (int64_t)0, T, E, units, ceil_log2(E), scratch, expanded, (int64_t)0,
@@ -348,7 +375,8 @@ extern "C" int hexa_route_from_lists(const int32_t* token_idx_list, const int32_
     }
     hipLaunchKernelGGL(route_from_lists_kernel, dim3(k), dim3(256), scan_lds_bytes(E), st, expert_idx_list, T, E,
                        route + L.counts, route + L.offsets, reinterpret_cast<int4*>(route + L.tile_info),
-                       route + L.tile_count, L.mt_ub);
+                       route + L.tile_count, L.mt_ub, reinterpret_cast<int4*>(route + L.tile_info_l),
+                       route + L.tile_count_l, L.mt_ub_l);
     HEXA_CHECK_LAUNCH("route_from_lists");
     return HEXA_OK;
 }

@@ -1,0 +1,318 @@
+// Routing front end for gfx950: gate projection, softmax + top-k + GShard auxiliary loss, and the
+// loss's backward through the softmax.  These are small HBM-/latency-bound kernels that replace a
+// dozen framework launches per MoE depth (fp32 cast, a skinny fp32 GEMM, softmax, top-k select + sort,
+// one-hot scatter, reductions).
+//
+// Reference: hexa_moe_cuda/hexa_moe/gates/top.py:17-19 (fp32 gate projection),
+//            hexa_moe_cuda/hexa_moe/impls/cascaded_moe.py:515-531 (noise, softmax, loss selection),
+//            hexa_moe_cuda/hexa_moe/impls/layers.py:476-484 (top-k), impls/losses.py:12-19 (GShard loss).
+#include "hexa_internal.h"
+
+namespace hexa {
+namespace {
+
+// ---- gate projection: logits[t][e] = sum_d x[t][d] * wg[e][d], fp32 accumulation ---------------------
+// 64 tokens per workgroup, one token per lane.  The model dimension is processed in chunks of 256:
+// the chunk of the 64 token rows and of 32 gate rows is staged in LDS with coalesced 16-byte loads;
+// each of the 4 wavefronts takes a quarter of the chunk, reads its token's pieces from LDS and the
+// gate row pieces as LDS broadcasts (one address for the whole wavefront), and the four partial sums
+// are folded through LDS in a fixed order.
+constexpr int GATE_EB = 32;    // experts per pass
+constexpr int GATE_DC = 256;   // model-dim chunk
+constexpr int GATE_XP = GATE_DC + 8;    // pitch of a staged token row, in elements (16 B of padding)
+constexpr int GATE_WP = GATE_DC + 4;    // pitch of a staged gate row, in floats
+
+template <typename T> struct Row8;   // 8 consecutive elements as floats
+template <> struct Row8<float> {
+    static __device__ __forceinline__ void load(const float* p, float (&v)[8]) {
+        const float4 a = reinterpret_cast<const float4*>(p)[0], b = reinterpret_cast<const float4*>(p)[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+};
+template <typename T16> struct Row8 {
+    static __device__ __forceinline__ void load(const T16* p, float (&v)[8]) {
+        union { uint4 u; T16 e[8]; } r;
+        r.u = *reinterpret_cast<const uint4*>(p);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (float)r.e[i];
+    }
+};
+
+template <typename T> constexpr int gate_smem_bytes() {
+    return 64 * GATE_XP * (int)sizeof(T) + GATE_EB * GATE_WP * 4 + 3 * 64 * (GATE_EB + 1) * 4;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gate_logits_kernel(float* __restrict__ logits, const T* __restrict__ x,
+                                                          const float* __restrict__ wg, int num_tokens, int d,
+                                                          int E) {
+    extern __shared__ __attribute__((aligned(16))) char gsm[];
+    T* sX = reinterpret_cast<T*>(gsm);
+    float* sW = reinterpret_cast<float*>(gsm + 64 * GATE_XP * sizeof(T));
+    float (*part)[64][GATE_EB + 1] = reinterpret_cast<float (*)[64][GATE_EB + 1]>(sW + GATE_EB * GATE_WP);
+    constexpr int VX = 16 / (int)sizeof(T);   // elements per 16-byte piece of a token row
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int t0 = blockIdx.x * 64;
+    const int t = t0 + lane;
+    for (int e0 = 0; e0 < E; e0 += GATE_EB) {
+        float acc[GATE_EB];
+#pragma unroll
+        for (int e = 0; e < GATE_EB; ++e) acc[e] = 0.f;
+        for (int d0 = 0; d0 < d; d0 += GATE_DC) {
+            const int dc = min(GATE_DC, d - d0);          // multiple of 8
+            __syncthreads();                               // previous chunk fully consumed
+            for (int i = tid; i < 64 * (dc / VX); i += 256) {
+                const int r = i / (dc / VX), c = i - r * (dc / VX);
+                uint4 v = make_uint4(0u, 0u, 0u, 0u);
+                if (t0 + r < num_tokens) v = *reinterpret_cast<const uint4*>(x + (size_t)(t0 + r) * d + d0 + c * VX);
+                *reinterpret_cast<uint4*>(sX + r * GATE_XP + c * VX) = v;
+            }
+            for (int i = tid; i < GATE_EB * (dc / 4); i += 256) {
+                const int r = i / (dc / 4), c = i - r * (dc / 4);
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (e0 + r < E) v = *reinterpret_cast<const float4*>(wg + (size_t)(e0 + r) * d + d0 + c * 4);
+                *reinterpret_cast<float4*>(sW + r * GATE_WP + c * 4) = v;
+            }
+            __syncthreads();
+            const int pieces = dc >> 3;
+            const int p0 = (pieces * wave) >> 2, p1 = (pieces * (wave + 1)) >> 2;
+            for (int pc = p0; pc < p1; ++pc) {
+                float xv[8];
+                Row8<T>::load(sX + lane * GATE_XP + pc * 8, xv);
+#pragma unroll
+                for (int e = 0; e < GATE_EB; ++e) {
+                    const float4 w0 = *reinterpret_cast<const float4*>(sW + e * GATE_WP + pc * 8);      // broadcast
+                    const float4 w1 = *reinterpret_cast<const float4*>(sW + e * GATE_WP + pc * 8 + 4);
+                    float a = acc[e];
+                    a = fmaf(xv[0], w0.x, a); a = fmaf(xv[1], w0.y, a); a = fmaf(xv[2], w0.z, a); a = fmaf(xv[3], w0.w, a);
+                    a = fmaf(xv[4], w1.x, a); a = fmaf(xv[5], w1.y, a); a = fmaf(xv[6], w1.z, a); a = fmaf(xv[7], w1.w, a);
+                    acc[e] = a;
+                }
+            }
+        }
+        if (wave > 0) {
+#pragma unroll
+            for (int e = 0; e < GATE_EB; ++e) part[wave - 1][lane][e] = acc[e];
+        }
+        __syncthreads();
+        if (wave == 0 && t < num_tokens) {
+#pragma unroll
+            for (int e = 0; e < GATE_EB; ++e) {
+                if (e0 + e < E)
+                    logits[(size_t)t * E + e0 + e] = ((acc[e] + part[0][lane][e]) + part[1][lane][e]) + part[2][lane][e];
+            }
+        }
+    }
+}
+
+// ---- softmax + top-k + per-workgroup loss partials ----------------------------------------------------
+// One token per lane, three passes over its logits row (max, sum of exp, scores + selection); the row
+// is tiny (E floats) and stays in L1/L2.  Ties go to the lower expert index.
+constexpr int MAX_TOPK = 8;
+
+constexpr int ROUTER_TB = 64;   // tokens (= lanes) per workgroup of the softmax/top-k kernel
+
+__global__ __launch_bounds__(ROUTER_TB) void router_fwd_kernel(float* __restrict__ scores, int32_t* __restrict__ idx,
+                                                         float* __restrict__ part_me, float* __restrict__ part_cnt,
+                                                         const float* __restrict__ logits,
+                                                         const float* __restrict__ noise, float noise_scale,
+                                                         int num_tokens, int E, int k) {
+    extern __shared__ float sh[];          // me[E] column sums of the wavefront, then cnt[E]
+    float* s_me = sh;
+    float* s_cnt = sh + E;
+    for (int i = threadIdx.x; i < 2 * E; i += blockDim.x) sh[i] = 0.f;
+    __syncthreads();
+    const int lane = threadIdx.x;
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool ok = t < num_tokens;
+    const float* lr = logits + (size_t)(ok ? t : 0) * E;
+    const float* nr = noise ? noise + (size_t)(ok ? t : 0) * E : nullptr;
+    float mx = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+        const float v = nr ? lr[e] + noise_scale * nr[e] : lr[e];
+        mx = fmaxf(mx, v);
+    }
+    float sum = 0.f;
+    for (int e = 0; e < E; ++e) {
+        const float v = nr ? lr[e] + noise_scale * nr[e] : lr[e];
+        sum += expf(v - mx);
+    }
+    const float inv = 1.0f / sum;
+    float best_v[MAX_TOPK];
+    int best_i[MAX_TOPK];
+#pragma unroll
+    for (int j = 0; j < MAX_TOPK; ++j) { best_v[j] = -INFINITY; best_i[j] = 0x7fffffff; }
+    for (int e = 0; e < E; ++e) {        // uniform trip count: every lane takes part in the reductions
+        const float v = nr ? lr[e] + noise_scale * nr[e] : lr[e];
+        const float sc = ok ? expf(v - mx) * inv : 0.f;
+        if (ok) scores[(size_t)t * E + e] = sc;
+        // insertion into the descending list; strict '>' keeps the lower index on ties
+        float cv = sc; int ci = e;
+#pragma unroll
+        for (int j = 0; j < MAX_TOPK; ++j) {
+            if (j < k && cv > best_v[j]) {
+                const float tv = best_v[j]; const int ti = best_i[j];
+                best_v[j] = cv; best_i[j] = ci; cv = tv; ci = ti;
+            }
+        }
+        // column sum over the wavefront: xor butterfly, a fixed summation tree
+        float r = sc;
+#pragma unroll
+        for (int m = 32; m > 0; m >>= 1) r += __shfl_xor(r, m);
+        if (lane == 0) s_me[e] = r;
+    }
+    if (ok) {
+#pragma unroll
+        for (int j = 0; j < MAX_TOPK; ++j)
+            if (j < k) idx[(size_t)t * k + j] = best_i[j];
+        atomicAdd(&s_cnt[best_i[0]], 1.0f);            // exact: at most 64 ones per counter
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        part_me[(size_t)blockIdx.x * E + e] = s_me[e];
+        part_cnt[(size_t)blockIdx.x * E + e] = s_cnt[e];
+    }
+}
+
+// me[e] = sum_t scores[t][e]; ce[e] = count[e] * E / T; l_aux = sum_e me[e]*ce[e] / T  (losses.py:12-19)
+__global__ __launch_bounds__(256) void router_loss_kernel(float* __restrict__ l_aux, float* __restrict__ me,
+                                                          float* __restrict__ ce, const float* __restrict__ part_me,
+                                                          const float* __restrict__ part_cnt, int nblocks,
+                                                          int num_tokens, int E) {
+    // per expert: 8 threads sum 8 contiguous ranges of the workgroup partials, then the 8 range sums
+    // are added in range order -- a fixed tree, independent of scheduling
+    extern __shared__ float sh[];          // [8][E] me, [8][E] cnt
+    float* s_m = sh;
+    float* s_c = sh + 8 * E;
+    __shared__ float red[256];
+    const int per = (nblocks + 7) / 8;
+    for (int i = threadIdx.x; i < 8 * E; i += 256) {
+        const int c = i / E, e = i - c * E;
+        const int b0 = c * per, b1 = min(nblocks, b0 + per);
+        float m = 0.f, n = 0.f;
+        for (int b = b0; b < b1; ++b) { m += part_me[(size_t)b * E + e]; n += part_cnt[(size_t)b * E + e]; }
+        s_m[i] = m;
+        s_c[i] = n;
+    }
+    __syncthreads();
+    float local = 0.f;
+    for (int e = threadIdx.x; e < E; e += 256) {
+        float m = 0.f, c = 0.f;
+        for (int j = 0; j < 8; ++j) { m += s_m[j * E + e]; c += s_c[j * E + e]; }
+        const float cev = c * ((float)E / (float)num_tokens);
+        me[e] = m;
+        ce[e] = cev;
+        local += m * cev;
+    }
+    red[threadIdx.x] = local;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if (threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *l_aux = red[0] / (float)num_tokens;
+}
+
+// d l_aux / d logits through the softmax: with c[e] = g * ce[e] / T,
+//   dlogits[t][e] = scores[t][e] * (c[e] - sum_e' scores[t][e'] * c[e'])
+__global__ __launch_bounds__(ROUTER_TB) void router_bwd_kernel(float* __restrict__ dlogits,
+                                                               const float* __restrict__ scores,
+                                                               const float* __restrict__ ce,
+                                                               const float* __restrict__ grad_l, int num_tokens, int E) {
+    extern __shared__ float s_c[];         // c[e] = g * ce[e] / T
+    const float g = *grad_l / (float)num_tokens;
+    for (int e = threadIdx.x; e < E; e += blockDim.x) s_c[e] = g * ce[e];
+    __syncthreads();
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= num_tokens) return;
+    const float* sr = scores + (size_t)t * E;
+    float* dr = dlogits + (size_t)t * E;
+    float dot = 0.f;
+    if ((E & 3) == 0) {
+        for (int e = 0; e < E; e += 4) {
+            const float4 v = *reinterpret_cast<const float4*>(sr + e);
+            dot += v.x * s_c[e] + v.y * s_c[e + 1] + v.z * s_c[e + 2] + v.w * s_c[e + 3];
+        }
+        for (int e = 0; e < E; e += 4) {
+            const float4 v = *reinterpret_cast<const float4*>(sr + e);
+            *reinterpret_cast<float4*>(dr + e) = make_float4(v.x * (s_c[e] - dot), v.y * (s_c[e + 1] - dot),
+                                                             v.z * (s_c[e + 2] - dot), v.w * (s_c[e + 3] - dot));
+        }
+    } else {
+        for (int e = 0; e < E; ++e) dot += sr[e] * s_c[e];
+        for (int e = 0; e < E; ++e) dr[e] = sr[e] * (s_c[e] - dot);
+    }
+}
+
+template <typename T>
+int launch_gate(dim3 grid, dim3 block, hipStream_t st, float* logits, const void* x, const float* wg, int num_tokens,
+                int d, int E) {
+    static bool attr_done = false;
+    constexpr int bytes = gate_smem_bytes<T>();
+    if (!attr_done) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(gate_logits_kernel<T>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
+            HEXA_FAIL(HEXA_ERR_LAUNCH, "hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d) failed", bytes);
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(gate_logits_kernel<T>, grid, block, bytes, st, logits, (const T*)x, wg, num_tokens, d, E);
+    HEXA_CHECK_LAUNCH("gate_logits");
+    return HEXA_OK;
+}
+
+}  // namespace
+}  // namespace hexa
+
+using namespace hexa;
+
+extern "C" int hexa_gate_logits(float* logits, const void* x, const float* wg, int T, int d, int E, int x_dt,
+                                void* stream) {
+    if (T < 0 || d < 1 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_logits: bad sizes T=%d d=%d E=%d", T, d, E);
+    if (T > 0 && (!logits || !x || !wg)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_logits: null pointer");
+    if (d % 8) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_gate_logits: model dim must be a multiple of 8 (got %d)", d);
+    if (T == 0) return HEXA_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid(div_up(T, 64)), block(256);
+    if (x_dt == HEXA_F32) return launch_gate<float>(grid, block, st, logits, x, wg, T, d, E);
+    if (x_dt == HEXA_BF16) return launch_gate<__bf16>(grid, block, st, logits, x, wg, T, d, E);
+    if (x_dt == HEXA_F16) return launch_gate<_Float16>(grid, block, st, logits, x, wg, T, d, E);
+    HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_logits: unknown element type");
+}
+
+extern "C" int hexa_router_ws_floats(int T, int E, int64_t* out) {
+    if (!out || T < 0 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_router_ws_floats: bad arguments");
+    *out = (int64_t)2 * (T > 0 ? div_up(T, ROUTER_TB) : 1) * E;
+    return HEXA_OK;
+}
+
+extern "C" int hexa_router_forward(float* scores, int32_t* idx, float* me, float* ce, float* l_aux,
+                                   const float* logits, const float* noise, float noise_scale, int T, int E, int k,
+                                   float* ws, void* stream) {
+    if (T < 1 || E < 1 || k < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_router_forward: bad sizes T=%d E=%d k=%d", T, E, k);
+    if (k > MAX_TOPK || k > E) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_router_forward: top_k must be <= min(E, %d)", MAX_TOPK);
+    if (!scores || !idx || !me || !ce || !l_aux || !logits || !ws) HEXA_FAIL(HEXA_ERR_ARG, "hexa_router_forward: null pointer");
+    if (E > 4096) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_router_forward: more than 4096 experts");
+    hipStream_t st = (hipStream_t)stream;
+    const int nb = div_up(T, ROUTER_TB);
+    float* part_me = ws;
+    float* part_cnt = ws + (size_t)nb * E;
+    hipLaunchKernelGGL(router_fwd_kernel, dim3(nb), dim3(ROUTER_TB), sizeof(float) * 2 * E, st, scores, idx, part_me,
+                       part_cnt, logits, noise, noise_scale, T, E, k);
+    HEXA_CHECK_LAUNCH("router_fwd");
+    hipLaunchKernelGGL(router_loss_kernel, dim3(1), dim3(256), sizeof(float) * 16 * E, st, l_aux, me, ce, part_me,
+                       part_cnt, nb, T, E);
+    HEXA_CHECK_LAUNCH("router_loss");
+    return HEXA_OK;
+}
+
+extern "C" int hexa_router_backward(float* dlogits, const float* scores, const float* ce, const float* grad_l_aux,
+                                    int T, int E, void* stream) {
+    if (T < 1 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_router_backward: bad sizes");
+    if (!dlogits || !scores || !ce || !grad_l_aux) HEXA_FAIL(HEXA_ERR_ARG, "hexa_router_backward: null pointer");
+    if (E > 8192) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_router_backward: more than 8192 experts");
+    hipLaunchKernelGGL(router_bwd_kernel, dim3(div_up(T, ROUTER_TB)), dim3(ROUTER_TB), sizeof(float) * E,
+                       (hipStream_t)stream, dlogits, scores, ce, grad_l_aux, T, E);
+    HEXA_CHECK_LAUNCH("router_bwd");
+    return HEXA_OK;
+}

@@ -13,6 +13,7 @@ HEXA_F32, HEXA_F16, HEXA_BF16 = 0, 1, 2
 HEXA_W_IN_OUT, HEXA_W_OUT_IN = 0, 1
 HEXA_ACT_NONE, HEXA_ACT_GELU = 0, 1
 HEXA_TILE_ROWS = 128
+HEXA_TILE_ROWS_L = 256
 HEXA_ROUTE_UNIT = 512
 
 _vp, _i, _i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
@@ -20,8 +21,10 @@ _vp, _i, _i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
 
 class RouteLayout(ctypes.Structure):
     _fields_ = [("counts", _i64), ("offsets", _i64), ("token_ids", _i64), ("expert_ids", _i64),
-                ("tile_count", _i64), ("tile_info", _i64), ("scratch", _i64), ("total_ints", _i64),
-                ("mt_ub", ctypes.c_int32), ("units", ctypes.c_int32)]
+                ("tile_count", _i64), ("tile_info", _i64), ("tile_count_l", _i64), ("tile_info_l", _i64),
+                ("scratch", _i64), ("total_ints", _i64),
+                ("mt_ub", ctypes.c_int32), ("mt_ub_l", ctypes.c_int32), ("units", ctypes.c_int32),
+                ("reserved", ctypes.c_int32)]
 
 
 # name -> (restype, argtypes); kept in one table so the export test can walk it
@@ -36,6 +39,10 @@ SIGNATURES = {
     "hexa_ess": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "hexa_fused_grad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "hexa_gelu_bwd": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),
+    "hexa_gate_logits": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "hexa_router_ws_floats": (_i, [_i, _i, ctypes.POINTER(_i64)]),
+    "hexa_router_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float, _i, _i, _i, _vp, _vp]),
+    "hexa_router_backward": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "hexa_last_error": (ctypes.c_char_p, []),
     "hexa_abi_version": (_i, []),
 }
@@ -57,7 +64,7 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.hexa_abi_version() != 2:
+    if lib.hexa_abi_version() != 3:
         raise RuntimeError("hexa_moe: libhexa_moe_hip.so has an unexpected ABI version")
     _lib = lib
     return lib

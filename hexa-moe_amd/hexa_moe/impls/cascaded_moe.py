@@ -33,7 +33,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from .. import ops
-from . import losses
+from . import losses, router
 from .layers import FusedMoE_Shared_CudaCore, MLP_Implement, simplified_extract_critical, topk_and_loss  # noqa: F401
 
 
@@ -125,6 +125,7 @@ class MoE_Cascaded(nn.Module):
         self.a2a_ffn_overlap_degree = a2a_ffn_overlap_degree
         self.use_2dh = use_2dh
         self.parallel_type = parallel_type
+        self.fused_router = True   # set False to route with the PyTorch formulation
         # One device holds every expert in full; a process group, if there is one, only replicates.
         self.world_size, self.local_rank = 1, 0
         if dist.is_available() and dist.is_initialized():
@@ -262,7 +263,12 @@ class MoE_Cascaded(nn.Module):
 
     # ---- forward -----------------------------------------------------------------------------------
     def _route(self, gate, x, top_k):
-        """gate -> (+noise) -> softmax -> top-k and the auxiliary loss (reference: cascaded_moe.py:515-531)."""
+        """gate -> (+noise) -> softmax -> top-k and the auxiliary loss (reference: cascaded_moe.py:515-531).
+        GPU inputs with the linear gate and the GShard loss take the fused kernels (impls/router.py)."""
+        if self.fused_router and router.fused_route_supported(gate, x, top_k, self.num_global_experts,
+                                                              self.is_gshard_loss):
+            return router.fused_route(gate, x, top_k, self.num_global_experts,
+                                      gate.gate_noise / self.num_global_experts, self.training)
         logits = gate(x)
         if self.training and gate.gate_noise > 0:
             logits_w_noise = logits + gate.gate_noise * torch.randn_like(logits) / self.num_global_experts

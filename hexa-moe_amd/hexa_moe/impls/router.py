@@ -1,0 +1,65 @@
+"""Fused routing front end: gate projection, softmax, top-k and the GShard loss as HIP kernels with
+autograd glue.  It computes what the reference's routing() closure computes
+(hexa_moe_cuda/hexa_moe/impls/cascaded_moe.py:515-531 with impls/layers.py:476-484 and
+impls/losses.py:12-19); MoE_Cascaded uses it for GPU inputs with the linear gate and the GShard loss and
+keeps the PyTorch formulation for everything else (cosine gate, load-importance loss, more than 8 slots).
+"""
+import torch
+
+from .. import ops
+
+
+class GateProjection(torch.autograd.Function):
+    """logits = x @ wg^T accumulated in fp32 whatever the tokens' type (the fp32 gate of
+    gates/top.py:17-19), without materialising an fp32 copy of x."""
+
+    @staticmethod
+    def forward(ctx, x, wg):
+        ctx.save_for_backward(x, wg)
+        return ops.gate_logits(x, wg.float())
+
+    @staticmethod
+    def backward(ctx, dlogits):
+        x, wg = ctx.saved_tensors
+        dx = dwg = None
+        if ctx.needs_input_grad[0]:
+            dx = (dlogits @ wg.float()).to(x.dtype)
+        if ctx.needs_input_grad[1]:
+            dwg = (dlogits.t() @ x.float()).to(wg.dtype)
+        return dx, dwg
+
+
+class RouterTopK(torch.autograd.Function):
+    """(idx [T,k] int32, l_aux) = top-k of softmax(logits + scale*noise) and the GShard loss."""
+
+    @staticmethod
+    def forward(ctx, logits, noise, noise_scale, top_k):
+        scores, idx, _me, ce, l_aux = ops.router_forward(logits, top_k, noise, noise_scale)
+        ctx.save_for_backward(scores, ce)
+        ctx.mark_non_differentiable(idx)
+        return idx, l_aux
+
+    @staticmethod
+    def backward(ctx, _didx, dl_aux):
+        scores, ce = ctx.saved_tensors
+        return ops.router_backward(scores, ce, dl_aux), None, None, None
+
+
+def fused_route_supported(gate, x, top_k, num_experts, is_gshard_loss):
+    from ..gates.top import LinearTopKGate
+    return (x.is_cuda and is_gshard_loss and isinstance(gate, LinearTopKGate) and 1 <= top_k <= min(8, num_experts)
+            and num_experts <= 4096 and x.shape[1] % 8 == 0
+            and x.dtype in (torch.float32, torch.float16, torch.bfloat16))
+
+
+def fused_route(gate, x, top_k, num_experts, noise_scale, training):
+    """Returns (indices [T,k] int32, l_aux)."""
+    w = gate.wg.weight
+    if gate.fp32_gate or x.dtype == torch.float32:
+        logits = GateProjection.apply(x, w)
+    else:   # a gate kept in the tokens' type: the framework's own linear, as in the reference
+        logits = gate(x).float()
+    noise = None
+    if training and noise_scale > 0:
+        noise = torch.randn_like(logits)
+    return RouterTopK.apply(logits, noise, float(noise_scale), int(top_k))

@@ -99,6 +99,14 @@ class Route:
     def tile_info(self):
         return self._part(self.layout.tile_info, self.k * self.layout.mt_ub * 4).view(self.k, self.layout.mt_ub, 4)
 
+    @property
+    def tile_count_l(self):
+        return self._part(self.layout.tile_count_l, self.k)
+
+    @property
+    def tile_info_l(self):
+        return self._part(self.layout.tile_info_l, self.k * self.layout.mt_ub_l * 4).view(self.k, self.layout.mt_ub_l, 4)
+
 
 class RouteWorkspace:
     """One int32 device buffer reused by every MoE depth of a model (the depth-shared cache of
@@ -224,3 +232,53 @@ def gelu_bwd(dy2, y1):
                _stream())
     _lib.check(rc, "hexa_gelu_bwd")
     return out
+
+
+def gate_logits(x, wg):
+    """logits[t][e] = sum_d x[t][d] * wg[e][d] with fp32 accumulation; wg fp32 [E, d] -> fp32 [T, E]."""
+    _dev(x, wg)
+    x = x.contiguous()
+    wg = wg.contiguous()
+    assert wg.dtype == torch.float32 and x.dim() == 2 and wg.shape[1] == x.shape[1]
+    T, d = x.shape
+    E = wg.shape[0]
+    logits = torch.empty(T, E, dtype=torch.float32, device=x.device)
+    rc = _call("gate_logits", _lib.load().hexa_gate_logits, _ptr(logits), _ptr(x), _ptr(wg), T, d, E, _dt(x), _stream())
+    _lib.check(rc, "hexa_gate_logits")
+    return logits
+
+
+def router_forward(logits, top_k, noise=None, noise_scale=0.0):
+    """softmax + top-k + GShard loss.  Returns scores [T,E] fp32, idx [T,k] int32, me [E], ce [E], l_aux []."""
+    import ctypes
+    _dev(logits, noise)
+    logits = logits.contiguous()
+    assert logits.dtype == torch.float32 and logits.dim() == 2
+    T, E = logits.shape
+    dev = logits.device
+    n = ctypes.c_int64()
+    _lib.check(_lib.load().hexa_router_ws_floats(T, E, ctypes.byref(n)), "hexa_router_ws_floats")
+    ws = torch.empty(int(n.value), dtype=torch.float32, device=dev)
+    scores = torch.empty(T, E, dtype=torch.float32, device=dev)
+    idx = torch.empty(T, top_k, dtype=torch.int32, device=dev)
+    stats = torch.empty(2 * E + 1, dtype=torch.float32, device=dev)   # me, ce, l_aux
+    me, ce, l_aux = stats[:E], stats[E:2 * E], stats[2 * E]
+    if noise is not None:
+        noise = noise.contiguous()
+        assert noise.dtype == torch.float32 and noise.shape == logits.shape
+    rc = _call("router_forward", _lib.load().hexa_router_forward, _ptr(scores), _ptr(idx), _ptr(me), _ptr(ce),
+               l_aux.data_ptr(), _ptr(logits), _ptr(noise), float(noise_scale), T, E, int(top_k), _ptr(ws), _stream())
+    _lib.check(rc, "hexa_router_forward")
+    return scores, idx, me, ce, l_aux
+
+
+def router_backward(scores, ce, grad_l_aux):
+    """d l_aux / d logits scaled by grad_l_aux (a 0-dim fp32 device tensor)."""
+    _dev(scores, ce, grad_l_aux)
+    T, E = scores.shape
+    g = grad_l_aux.to(torch.float32).contiguous()
+    dlogits = torch.empty_like(scores)
+    rc = _call("router_backward", _lib.load().hexa_router_backward, _ptr(dlogits), _ptr(scores), _ptr(ce), _ptr(g), T, E,
+               _stream())
+    _lib.check(rc, "hexa_router_backward")
+    return dlogits

@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define HEXA_ABI_VERSION 2
+#define HEXA_ABI_VERSION 3
 
 /* element types */
 #define HEXA_F32 0
@@ -43,6 +43,8 @@ extern "C" {
 /* Rows per row-tile of the gathered-row kernels; the routing pass emits one tile record per
  * HEXA_TILE_ROWS rows of every (slot, expert) segment. */
 #define HEXA_TILE_ROWS 128
+/* A second set of records with twice as many rows per tile, for the large-tile kernels. */
+#define HEXA_TILE_ROWS_L 256
 /* Tokens handled by one wavefront in the routing pass. */
 #define HEXA_ROUTE_UNIT 512
 
@@ -56,16 +58,19 @@ extern "C" {
  *   expert_ids [k][T]        expert of each list position (the reference's expert_idx_list)
  *   tile_count [k]           number of row tiles of the slot
  *   tile_info  [k][mt_ub][4] {expert, first list position, rows (<=HEXA_TILE_ROWS), 0}
+ *   tile_count_l [k], tile_info_l [k][mt_ub_l][4]   the same with HEXA_TILE_ROWS_L rows per tile
  *   scratch    [k][units][E] per-wavefront histograms of the routing pass
  * The buffer may be shared by all MoE depths of a model (sized for the largest T*k): its contents
  * are rebuilt by hexa_route_build for each depth and reused by that depth's forward and backward
  * operators.
  * ---------------------------------------------------------------------------------------------- */
 typedef struct hexa_route_layout {
-    int64_t counts, offsets, token_ids, expert_ids, tile_count, tile_info, scratch;
+    int64_t counts, offsets, token_ids, expert_ids, tile_count, tile_info, tile_count_l, tile_info_l, scratch;
     int64_t total_ints; /* size of the blob in int32 elements */
     int32_t mt_ub;      /* row-tile upper bound per slot: T/HEXA_TILE_ROWS + E                      */
+    int32_t mt_ub_l;    /* the same for HEXA_TILE_ROWS_L                                            */
     int32_t units;      /* wavefront units per slot: ceil(T/HEXA_ROUTE_UNIT)                        */
+    int32_t reserved;
 } hexa_route_layout;
 
 int hexa_route_layout_get(int num_tokens, int top_k, int num_experts, hexa_route_layout* out);
@@ -150,6 +155,27 @@ int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y, const void
 /* Elementwise backward of the fused GELU: dy1 = dy2 * gelu'(y1), n elements of type dt.  The
  * reference evaluates act' with torch.autograd.functional.jacobian (impls/layers.py:281-283,427). */
 int hexa_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, void* stream);
+
+/* ---- routing front end (fused; the PyTorch path of the host code stays available) ----------------
+ * Gate projection logits[t][e] = sum_d x[t][d]*wg[e][d] with fp32 accumulation; x is F32/F16/BF16,
+ * wg fp32 [E][d], d a multiple of 8.  Replaces LinearTopKGate.forward with fp32_gate (gates/top.py:17-19:
+ * a cast of x to fp32 plus a skinny fp32 GEMM). */
+int hexa_gate_logits(float* logits, const void* x, const float* wg, int num_tokens, int model_dim,
+                     int num_experts, int x_dt, void* stream);
+
+/* softmax(logits + noise_scale*noise) -> scores [T][E]; top-k expert ids idx [T][k] (int32, descending
+ * score, ties to the lower id); me[e] = sum_t scores, ce[e] = (E/T)*#{t: top-1 = e}; l_aux =
+ * sum_e me*ce / T (the GShard loss).  noise may be NULL.  ws: hexa_router_ws_floats() floats.
+ * Replaces routing() + simplified_extract_critical + gshard_loss
+ * (impls/cascaded_moe.py:515-531, impls/layers.py:476-484, impls/losses.py:12-19). */
+int hexa_router_ws_floats(int num_tokens, int num_experts, int64_t* out);
+int hexa_router_forward(float* scores, int32_t* idx, float* me, float* ce, float* l_aux, const float* logits,
+                        const float* noise, float noise_scale, int num_tokens, int num_experts, int top_k,
+                        float* ws, void* stream);
+/* dlogits = d l_aux / d logits * (*grad_l_aux), through the softmax (ce is treated as a constant, as
+ * in the reference where the one-hot mask carries no gradient). */
+int hexa_router_backward(float* dlogits, const float* scores, const float* ce, const float* grad_l_aux,
+                         int num_tokens, int num_experts, void* stream);
 
 const char* hexa_last_error(void);
 int hexa_abi_version(void);

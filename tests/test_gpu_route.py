@@ -51,6 +51,13 @@ def test_route_build_matches_oracle(dev, T, E, k, skew, empty, as_i64):
         assert int(ntile[s]) == len(want)
         got = [tuple(int(v) for v in row) for row in tiles[s, :len(want)]]
         assert got == want
+        want_l = []
+        for e in range(E):
+            c, o = int(counts[s, e]), int(offsets[s, e])
+            for j in range(0, c, 256):
+                want_l.append((e, o + j, min(256, c - j), 0))
+        assert int(route.tile_count_l[s]) == len(want_l)
+        assert [tuple(int(v) for v in row) for row in route.tile_info_l.cpu()[s, :len(want_l)]] == want_l
     if skew == "zipf":
         assert int((counts.sum(0) == 0).sum()) >= empty
 

@@ -33,7 +33,7 @@ def test_header_symbols_are_exported():
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in include/hexa_moe_hip.h but not exported"
     assert declared == set(_lib.SIGNATURES), "ctypes table and header disagree"
-    assert lib.hexa_abi_version() == 2
+    assert lib.hexa_abi_version() == 3
 
 
 def test_abi_argument_errors_without_a_gpu():
@@ -45,7 +45,9 @@ def test_abi_argument_errors_without_a_gpu():
     assert lib.hexa_token_count(None, None, None, 4, 2, 1, None, None) == -1
     L = _lib.route_layout(18432, 2, 32)
     assert L.mt_ub == 18432 // 128 + 32 and L.units == 36 and L.tile_info % 4 == 0
-    parts = [L.counts, L.offsets, L.token_ids, L.expert_ids, L.tile_count, L.tile_info, L.scratch, L.total_ints]
+    assert L.mt_ub_l == 18432 // 256 + 32 and L.tile_info_l % 4 == 0
+    parts = [L.counts, L.offsets, L.token_ids, L.expert_ids, L.tile_count, L.tile_info, L.tile_count_l, L.tile_info_l,
+             L.scratch, L.total_ints]
     assert parts == sorted(parts)
 
 

@@ -48,7 +48,8 @@ extern "C" int hexa_esmm(void* out, const void* x, const void* w, const void* bi
     if (w_layout != HEXA_W_IN_OUT && w_layout != HEXA_W_OUT_IN) HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: bad w_layout %d", w_layout);
     if (!is_dt(x_dt) || !is_dt(w_dt) || !is_dt(out_dt) || (bias && !is_dt(bias_dt)))
         HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: unknown element type");
-    if (act != HEXA_ACT_NONE && act != HEXA_ACT_GELU) HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: unknown activation %d", act);
+    if (act != HEXA_ACT_NONE && act != HEXA_ACT_GELU && act != HEXA_ACT_GELU_BWD)
+        HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: unknown activation %d", act);
     if (act != HEXA_ACT_NONE && (!out_act || m2s || accumulate))
         HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: a fused activation needs out_act, m2s == 0 and accumulate == 0");
     if (T == 0) return HEXA_OK;

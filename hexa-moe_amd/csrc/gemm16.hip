@@ -232,7 +232,8 @@ __global__ __launch_bounds__(NT, 2) void esmm16_kernel(EsmmK p) {
                 const int tok = sTok[row];
                 if (tok < 0) continue;
                 const size_t idx = ((size_t)p.out_slot_rows * s + tok) * N + col;
-                const float val = acc[i][j][v] + bv;
+                float val = acc[i][j][v] + bv;
+                if (p.act == HEXA_ACT_GELU_BWD) val *= gelu_grad_erf(load_as_f(p.out_act, idx, p.out_dt));
                 store_out(p.out, idx, val, p.out_dt, accumulate);
                 if (p.act == HEXA_ACT_GELU) store_out(p.out_act, idx, gelu_erf(val), p.out_dt, false);
             }

@@ -164,7 +164,8 @@ __global__ __launch_bounds__(NT, 2) void esmm32_kernel(EsmmK p) {
                 const int t = sTok[row];
                 if (t < 0) continue;
                 const size_t idx = ((size_t)p.out_slot_rows * s + t) * N + col;
-                const float val = acc[i][j][v] + bv;
+                float val = acc[i][j][v] + bv;
+                if (p.act == HEXA_ACT_GELU_BWD) val *= gelu_grad_erf(p.out_act[idx]);
                 p.out[idx] = p.accumulate ? p.out[idx] + val : val;
                 if (p.act == HEXA_ACT_GELU) p.out_act[idx] = gelu_erf(val);
             }

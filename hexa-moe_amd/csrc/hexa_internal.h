@@ -74,6 +74,8 @@ struct EssArgs {
 int launch_esmm16(const EsmmArgs& a, hipStream_t s);
 int launch_esmm32(const EsmmArgs& a, hipStream_t s);
 bool esmm16_dma_supported(const EsmmArgs& a);
+bool esmm16_persist_supported(const EsmmArgs& a);
+int launch_esmm16_persist(const EsmmArgs& a, int tile, hipStream_t st);
 int launch_esmm16_dma(const EsmmArgs& a, hipStream_t s);
 bool dma_path_enabled();
 bool estmm16_dma_supported(const EstmmArgs& a);
@@ -87,6 +89,11 @@ int launch_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int d
 // ---- small device helpers -------------------------------------------------------------------
 __device__ __forceinline__ float gelu_erf(float x) {
     return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+}
+
+// gelu'(x) = Phi(x) + x * phi(x), erf form
+__device__ __forceinline__ float gelu_grad_erf(float x) {
+    return 0.5f * (1.0f + erff(x * 0.70710678118654752440f)) + x * 0.39894228040143267794f * expf(-0.5f * x * x);
 }
 
 template <typename T> struct Cvt;

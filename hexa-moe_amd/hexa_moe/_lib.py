@@ -11,7 +11,7 @@ LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "lib", "libhexa_moe_hip.so
 
 HEXA_F32, HEXA_F16, HEXA_BF16 = 0, 1, 2
 HEXA_W_IN_OUT, HEXA_W_OUT_IN = 0, 1
-HEXA_ACT_NONE, HEXA_ACT_GELU = 0, 1
+HEXA_ACT_NONE, HEXA_ACT_GELU, HEXA_ACT_GELU_BWD = 0, 1, 2
 HEXA_TILE_ROWS = 128
 HEXA_TILE_ROWS_L = 256
 HEXA_ROUTE_UNIT = 512

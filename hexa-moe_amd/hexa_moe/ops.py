@@ -152,8 +152,9 @@ def route_from_lists(token_idx_list, expert_idx_list, T, k, num_experts, blob=No
     return Route(blob, T, k, num_experts)
 
 
-def esmm(x, w, bias, route, m2s, w_layout, out=None, out_dtype=None, accumulate=False, gelu=False):
-    """out[(s),t] (+)= x[(s),t] @ W[e] + bias[e].  Returns out, or (out, gelu(out)) when gelu=True."""
+def esmm(x, w, bias, route, m2s, w_layout, out=None, out_dtype=None, accumulate=False, gelu=False, gelu_bwd_of=None):
+    """out[(s),t] (+)= x[(s),t] @ W[e] + bias[e].  Returns out, or (out, gelu(out)) when gelu=True.
+    gelu_bwd_of=y1 multiplies the result by gelu'(y1) (y1 of out's shape and dtype)."""
     _dev(x, w, bias, out)
     T, k, E = route.T, route.k, route.E
     x = x.contiguous()
@@ -170,16 +171,22 @@ def esmm(x, w, bias, route, m2s, w_layout, out=None, out_dtype=None, accumulate=
         out = torch.empty((T, out_dim) if m2s else (k, T, out_dim), dtype=out_dtype, device=x.device)
     assert out.is_contiguous() and tuple(out.shape) == ((T, out_dim) if m2s else (k, T, out_dim))
     out_act = torch.empty_like(out) if gelu else None
+    act = _lib.HEXA_ACT_GELU if gelu else _lib.HEXA_ACT_NONE
+    if gelu_bwd_of is not None:
+        assert not gelu and not m2s and not accumulate
+        out_act = gelu_bwd_of.contiguous()
+        assert out_act.shape == out.shape and out_act.dtype == out.dtype
+        act = _lib.HEXA_ACT_GELU_BWD
     # scratch for summing the slots in one launch (see hexa_esmm in include/hexa_moe_hip.h)
     slot_ws = torch.empty((k - 1, T, out_dim), dtype=out.dtype, device=out.device) if (m2s and k > 1) else None
     if bias is not None:
         bias = bias.contiguous()
     label = f"esmm[{in_dim}->{out_dim},{'w_in_out' if w_layout == _lib.HEXA_W_IN_OUT else 'w_out_in'}" \
-            f"{',sum_slots' if m2s else ''}{',gelu' if gelu else ''}]"
+            f"{',sum_slots' if m2s else ''}{',gelu' if gelu else ''}{',gelu_bwd' if gelu_bwd_of is not None else ''}]"
     rc = _call(label, _lib.load().hexa_esmm, _ptr(out), _ptr(x), _ptr(w), _ptr(bias), _ptr(route.blob),
                int(bool(m2s)), int(w_layout), int(bool(accumulate)), T, k, in_dim, out_dim, E, _dt(x), _dt(w),
                _dt(bias) if bias is not None else 0, _dt(out),
-               _lib.HEXA_ACT_GELU if gelu else _lib.HEXA_ACT_NONE, _ptr(out_act), _ptr(slot_ws), _stream())
+               act, _ptr(out_act), _ptr(slot_ws), _stream())
     _lib.check(rc, "hexa_esmm")
     return (out, out_act) if gelu else out
 

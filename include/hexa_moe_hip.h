@@ -33,6 +33,7 @@ extern "C" {
 /* epilogue activations of hexa_esmm */
 #define HEXA_ACT_NONE 0
 #define HEXA_ACT_GELU 1 /* out_act = gelu_erf(out), written next to the pre-activation `out`        */
+#define HEXA_ACT_GELU_BWD 2 /* out = (x.W) * gelu'(y1) with y1 READ from out_act (same shape as out)   */
 
 /* return codes */
 #define HEXA_OK 0
@@ -110,6 +111,8 @@ int hexa_route_from_lists(const int32_t* token_idx_list, const int32_t* expert_i
  * bias and out must be F32: true-fp32 MFMA path) or F16/BF16 (w may be the same 16-bit type or F32,
  * fp32 accumulation; out may be that 16-bit type or F32).  accumulate != 0 adds into `out`.
  * act == HEXA_ACT_GELU additionally writes gelu(out) to out_act (same shape/dtype as out; m2s == 0).
+ * act == HEXA_ACT_GELU_BWD multiplies the result by gelu'(y1), y1 read from out_act (same shape/dtype
+ * as out; m2s == 0, no accumulate): the backward ESMM dy1 = (dy.W2^T) * act'(y1) in one pass.
  * Dimension granularity: in and out multiples of 8 (16-bit) / 4 (fp32).
  * slot_ws (may be NULL) is scratch for m2s != 0 with top_k > 1: (top_k-1)*T*out elements of out_dt.
  * With it, all slots run in ONE launch (slot 0 writes `out`, the others write slot_ws) followed by a

@@ -171,6 +171,28 @@ def test_gelu_bwd(dev, dtype):
     assert_close(got, want, 2e-6 if dtype == F32 else TOL[dtype], "gelu_bwd")
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16, F16])
+@pytest.mark.parametrize("d_in,d_out", [(96, 200), (200, 96), (384, 1536)])
+def test_esmm_fused_gelu_bwd(dev, dtype, d_in, d_out):
+    """dy1 = (dy . W^T) * gelu'(y1) in one ESMM (weights stored [E, out, in] as in the backward)."""
+    from hexa_moe import _lib, ops
+    T, E, k = 900, 6, 2
+    g = gen(d_in)
+    routing = make_routing(T, E, k, seed=31)
+    x, W, _ = make_linear(T, d_in, d_out, E, k, seed=32, dtype=dtype, m2s=False)
+    y1 = (torch.randn(k, T, d_out, generator=g) * 2).to(dtype)
+    _, offsets, token_ids = O.route_build(routing, E)
+    rd = _ref_dtype(dtype)
+    lin = O.esmm(x.to(rd), W.to(rd), None, token_ids, offsets, False)
+    yr = y1.double().requires_grad_(True)
+    (want,) = torch.autograd.grad(torch.nn.functional.gelu(yr), yr, lin.double())
+    route = ops.route_build(routing.to(dev), E)
+    for lay, Wd in ((_lib.HEXA_W_OUT_IN, W.transpose(1, 2).contiguous()), (_lib.HEXA_W_IN_OUT, W)):
+        got = ops.esmm(x.to(dev), Wd.to(dev), None, route, False, lay, gelu_bwd_of=y1.to(dev))
+        torch.cuda.synchronize()
+        assert_close(got, want, TOL[dtype], "esmm * gelu'")
+
+
 def test_reference_style_ops(dev):
     """The five operator names of the reference extension, called the way impls/layers.py calls them."""
     import hexa_moe_cuda

@@ -28,6 +28,16 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
 T, D, H, E, K_TOP = 18432, 384, 1536, 32, 2
 SEED = 1235
 
+# HBM bytes per launch (fetch + write) of the matmul kernels on this workload, from rocprofv3 FETCH_SIZE /
+# WRITE_SIZE counter passes scaled by a plain elementwise kernel of known size (--calibrate-copy); the
+# commands and the per-kernel figures are in profiles/*.hbm_traffic.txt.  Keys are the per-op labels.
+MEASURED_TRAFFIC_BYTES = {
+    "estmm[1536x384]": 373.3e6,
+    "esmm[1536->384,w_in_out,sum_slots]": 314.6e6,
+    "esmm[384->1536,w_out_in,gelu]": 409.9e6,       # average over the two launches of this kernel
+    "esmm[384->1536,w_out_in,gelu_bwd]": 409.9e6,   # (forward with GELU, backward with GELU')
+}
+
 
 def make_module_and_inputs(dev):
     """MoE_Cascaded with one MoE depth at the benchmark shape.  Expert parameters are bf16, the gate is
@@ -68,6 +78,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-events", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run a plain elementwise kernel over 256 MiB in / 256 MiB out (for scaling HBM counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (data-centric mode, no expert or model sharding, no "
@@ -91,6 +103,14 @@ def main():
         y, l_aux = m(0, x)
         torch.autograd.backward([y, l_aux], [dy, one])
         return y, m.dispatch_params.indices_
+
+    if args.calibrate_copy:   # known traffic: 2^27 bf16 read + 2^27 bf16 written per launch
+        src = torch.ones(1 << 27, dtype=torch.bfloat16, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()
@@ -138,7 +158,7 @@ def main():
         d = kernels[dom]
         if d["bound"] == "mfma":
             roofline = {"kernel": dom, "bound": "mfma", "achieved": d["tflops"], "peak": PEAK_BF16_TFLOPS,
-                        "unit": "TFLOP/s", "frac": d["frac"], "traffic": None}
+                        "unit": "TFLOP/s", "frac": d["frac"], "traffic": MEASURED_TRAFFIC_BYTES.get(dom)}
         else:
             roofline = {"kernel": dom, "bound": "hbm", "achieved": d["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                         "frac": d["frac"], "traffic": None}

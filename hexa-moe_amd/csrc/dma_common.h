@@ -15,12 +15,14 @@ constexpr int BK = 32;
 
 // WR x WF wavefronts, each computing RB x FB blocks of 32x32 (RB blocks along the rows, FB along the
 // fast output dimension).  MINW = wavefronts per SIMD the register budget is sized for.
-template <int WR_, int WF_, int RB_, int FB_, int STAGES_, int MINW_>
+// BKC = contraction indices per stage (32, or 64 for the ESMM kernels: whole 128-byte lines of a row).
+template <int WR_, int WF_, int RB_, int FB_, int STAGES_, int MINW_, int BKC_ = 32>
 struct Cfg {
     static constexpr int WR = WR_, WF = WF_, RB = RB_, FB = FB_, NW = WR_ * WF_, NT = 64 * NW, MINW = MINW_;
-    static constexpr int BM = 32 * RB_ * WR_, BN = 32 * FB_ * WF_, STAGES = STAGES_;
-    static constexpr int R_BYTES = BM * BK * 2, F_BYTES = BN * BK * 2, STAGE_BYTES = R_BYTES + F_BYTES;
-    static constexpr int R_COPIES = BM / 16, F_COPIES = BN / 16;      // wavefront copies per stage
+    static constexpr int BM = 32 * RB_ * WR_, BN = 32 * FB_ * WF_, STAGES = STAGES_, BKC = BKC_;
+    static constexpr int R_BYTES = BM * BKC * 2, F_BYTES = BN * BKC * 2, STAGE_BYTES = R_BYTES + F_BYTES;
+    static constexpr int R_COPIES = R_BYTES / 1024, F_COPIES = F_BYTES / 1024;   // wavefront copies per stage
+    static_assert(BKC == 32 || BKC == 64, "32 or 64 contraction indices per stage");
     static constexpr int R_CPW = R_COPIES / NW, F_CPW = F_COPIES / NW, CPW = R_CPW + F_CPW;
     static constexpr int STAGE_AREA = STAGES * STAGE_BYTES;
     static_assert(R_COPIES % NW == 0 && F_COPIES % NW == 0, "copies must divide evenly over the wavefronts");
@@ -32,6 +34,11 @@ using CfgM = Cfg<2, 2, 4, 2, 3, 2>;   // 256 x 128, 4 wavefronts of 128x64
 using CfgX = Cfg<2, 2, 4, 4, 3, 1>;   // 256 x 256, 4 wavefronts of 128x128
 using CfgX8 = Cfg<2, 4, 4, 2, 3, 2>;  // 256 x 256, 8 wavefronts of 128x64
 using CfgX16 = Cfg<4, 4, 2, 2, 3, 4>; // 256 x 256, 16 wavefronts of 64x64
+using CfgS2 = Cfg<2, 2, 2, 2, 2, 4>;  // 128 x 128, 2 stages, 4 workgroups per CU (128 registers)
+using CfgS3 = Cfg<2, 2, 2, 2, 3, 3>;  // 128 x 128, 3 stages, 3 workgroups per CU (168 registers)
+using CfgS64 = Cfg<2, 2, 2, 2, 2, 2, 64>;  // 128 x 128, 64 contraction indices per stage, 2 stages
+using CfgL64 = Cfg<4, 2, 2, 2, 2, 4, 64>;  // 256 x 128, 8 wavefronts, 64 per stage, 2 stages
+using CfgW = Cfg<2, 4, 2, 3, 3, 2>;   // 128 x 384, 8 wavefronts of 64x96: one tile spans a 384-wide result
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
@@ -93,12 +100,17 @@ __device__ __forceinline__ long logical_tile(int group) {
 
 // ---- fragment reads ---------------------------------------------------------------------------------
 // KC tile: 32x16 fragment (rows row0..row0+31, k = 16*ks..16*ks+15): lane holds row l%32, 8 k.
-template <typename V>
+// A row holds KD contraction indices (2*KD bytes, KD/8 pieces of 16 bytes); piece p of row r sits at
+// position p ^ kc_swizzle(r): rows that share a 256-byte span of LDS get different bank groups.
+template <int KD> __device__ __forceinline__ int kc_swizzle(int row) {
+    return KD == 32 ? (row >> 2) & 3 : (row >> 1) & 7;
+}
+template <typename V, int KD = 32>
 __device__ __forceinline__ V frag_kc(const char* tile, int row0, int ks, int lane) {
     const int row = row0 + (lane & 31);
     const int kch = ks * 2 + (lane >> 5);
-    const int pos = kch ^ ((row >> 2) & 3);
-    return *reinterpret_cast<const V*>(tile + row * 64 + pos * 16);
+    const int pos = kch ^ kc_swizzle<KD>(row);
+    return *reinterpret_cast<const V*>(tile + row * (2 * KD) + pos * 16);
 }
 
 // LDS reads issued as inline assembly: the compiler cannot see that they touch LDS, so it does not
@@ -140,17 +152,18 @@ __device__ __forceinline__ V frag_ks(const char* tile, int col0, int ks, int lan
 }
 
 // ---- copy-source helpers: which global piece does this lane fetch for wavefront copy `c` ------------
-// KC operand: copy c covers tile rows 16c..16c+15.
-__device__ __forceinline__ void kc_lane(int c, int lane, int& row, int& kc) {
-    row = 16 * c + (lane >> 2);
-    kc = (lane & 3) ^ ((row >> 2) & 3);
+// KC operand with KD contraction indices per row: copy c covers 512/KD tile rows.
+template <int KD = 32> __device__ __forceinline__ void kc_lane(int c, int lane, int& row, int& kc) {
+    constexpr int PPR = KD / 8;              // 16-byte pieces per row
+    row = (64 / PPR) * c + lane / PPR;
+    kc = (lane % PPR) ^ kc_swizzle<KD>(row);
 }
 // KS operand of width W: copy c covers 512/W k rows; returns the k row and the column piece.
 template <int W> __device__ __forceinline__ void ks_lane(int c, int lane, int& kk, int& ch) {
-    constexpr int PPR = W / 8;               // 16-byte pieces per k row
-    constexpr int RPC = 64 / PPR;            // k rows per wavefront copy
-    kk = RPC * c + lane / PPR;
-    ch = (lane % PPR) ^ ((kk & 3) << 2);
+    constexpr int PPR = W / 8;               // 16-byte pieces per k row (any multiple of 4)
+    const int piece = 64 * c + lane;
+    kk = piece / PPR;
+    ch = (piece - kk * PPR) ^ ((kk & 3) << 2);
 }
 
 template <int A, int B> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[A][B]) {
@@ -164,11 +177,14 @@ template <int A, int B> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[A
 
 // acc[j][i]: j = 32-wide block of the fast output dimension (operand "F"), i = 32-row block ("R").
 template <typename V, int NA, int NB> __device__ __forceinline__ void lds_fence_all(V (&a)[NA], V (&b)[NB]) {
-    // one s_waitcnt that every fragment "passes through" (see lds_fence)
-    if constexpr (NA == 2 && NB == 2) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]));
-    else if constexpr (NA == 2 && NB == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
-    else if constexpr (NA == 4 && NB == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
-    else static_assert(NA == 2 && NB == 2, "unsupported fragment counts");
+    // The wait carries no operands; every fragment is then passed through an empty statement placed
+    // BEHIND the wait, so a register copy the compiler makes for it reads completed data, and the
+    // MFMAs that consume the fragments cannot be scheduled ahead of the wait.
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < NA; ++i) asm volatile("" : "+v"(a[i]));
+#pragma unroll
+    for (int i = 0; i < NB; ++i) asm volatile("" : "+v"(b[i]));
 }
 
 template <typename TC, typename C, bool F_KS, bool R_KS>
@@ -177,14 +193,14 @@ __device__ __forceinline__ void mma_stage(const char* tileR, const char* tileF, 
     using V = typename Mfma<TC>::V;
     constexpr int RW = 32 * C::RB, FW = 32 * C::FB;   // rows / columns per wavefront
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
+    for (int ks = 0; ks < C::BKC / 16; ++ks) {
         V f[C::FB], r[C::RB];
 #pragma unroll
         for (int j = 0; j < C::FB; ++j)
-            f[j] = F_KS ? frag_ks<V, C::BN>(tileF, wf * FW + j * 32, ks, lane) : frag_kc<V>(tileF, wf * FW + j * 32, ks, lane);
+            f[j] = F_KS ? frag_ks<V, C::BN>(tileF, wf * FW + j * 32, ks, lane) : frag_kc<V, C::BKC>(tileF, wf * FW + j * 32, ks, lane);
 #pragma unroll
         for (int i = 0; i < C::RB; ++i)
-            r[i] = R_KS ? frag_ks<V, C::BM>(tileR, wr * RW + i * 32, ks, lane) : frag_kc<V>(tileR, wr * RW + i * 32, ks, lane);
+            r[i] = R_KS ? frag_ks<V, C::BM>(tileR, wr * RW + i * 32, ks, lane) : frag_kc<V, C::BKC>(tileR, wr * RW + i * 32, ks, lane);
         if (F_KS || R_KS) lds_fence_all(f, r);
 #pragma unroll
         for (int j = 0; j < C::FB; ++j)

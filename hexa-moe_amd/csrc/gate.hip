@@ -1,0 +1,285 @@
+// The gate's linear layer in fp32 on the matrix cores (v_mfma_f32_32x32x2_f32: fp32 multiply, fp32
+// accumulate), forward and backward, for token tensors of any supported type:
+//   logits[t][e] = sum_c x[t][c] * wg[e][c]                 (gate_fwd_kernel)
+//   dx[t][c]     = sum_e dlogits[t][e] * wg[e][c]           (gate_dx_kernel)
+//   dwg[e][c]    = sum_t dlogits[t][e] * x[t][c]            (gate_dwg_kernel + gate_dwg_reduce_kernel)
+// These are skinny products (E is a few dozen), HBM-bound on the token tensor; operands go from
+// global memory straight to registers.  The MFMA takes ONE contraction index per lane (lane l: row or
+// column l%32, index l/32), and which two indices one MFMA pairs is free as long as both operands
+// agree -- so a lane loads 8 (or 16) consecutive contraction indices in one go and feeds them to
+// consecutive MFMAs.  Where the fast output dimension is the token/gate row (dx, dwg), lane n owns 4
+// consecutive columns of a 128-column group, one accumulator per column offset: loads and stores
+// are whole 8- or 16-byte pieces.
+//
+// Replaces LinearTopKGate.forward with fp32_gate (gates/top.py:17-19: a cast of x to fp32 plus a
+// skinny fp32 GEMM) and what autograd derives from it.
+#include "hexa_internal.h"
+
+namespace hexa {
+namespace {
+
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+constexpr int GT = 32;          // tokens per workgroup (forward, dx)
+constexpr int DWG_TB = 64;      // tokens per workgroup (dwg)
+
+__device__ __forceinline__ f32x16 zero16() {
+    f32x16 z;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) z[v] = 0.f;
+    return z;
+}
+
+// N consecutive elements (N = 4 or 8) as floats; zeros when !ok
+template <typename T, int N> struct LoadN {   // 16-bit types
+    static __device__ __forceinline__ void run(const T* p, bool ok, float (&o)[N]) {
+        union { unsigned u[N / 2]; T h[N]; } v;
+        if (N == 8) {
+            const uint4 w = ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0u, 0u, 0u, 0u);
+            v.u[0] = w.x; v.u[1] = w.y; v.u[N / 2 - 2] = w.z; v.u[N / 2 - 1] = w.w;
+        } else {
+            const uint2 w = ok ? *reinterpret_cast<const uint2*>(p) : make_uint2(0u, 0u);
+            v.u[0] = w.x; v.u[1] = w.y;
+        }
+#pragma unroll
+        for (int i = 0; i < N; ++i) o[i] = (float)v.h[i];
+    }
+};
+template <int N> struct LoadN<float, N> {
+    static __device__ __forceinline__ void run(const float* p, bool ok, float (&o)[N]) {
+#pragma unroll
+        for (int q = 0; q < N; q += 4) {
+            const float4 v = ok ? *reinterpret_cast<const float4*>(p + q) : make_float4(0.f, 0.f, 0.f, 0.f);
+            o[q] = v.x; o[q + 1] = v.y; o[q + 2] = v.z; o[q + 3] = v.w;
+        }
+    }
+};
+template <typename T> __device__ __forceinline__ void store4(T* p, float a, float b, float c, float d);
+template <> __device__ __forceinline__ void store4<float>(float* p, float a, float b, float c, float d) {
+    *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
+}
+template <typename T16> __device__ __forceinline__ void store4(T16* p, float a, float b, float c, float d) {
+    union { uint2 u; T16 h[4]; } v;
+    v.h[0] = (T16)a; v.h[1] = (T16)b; v.h[2] = (T16)c; v.h[3] = (T16)d;
+    *reinterpret_cast<uint2*>(p) = v.u;
+}
+
+// ---- forward: 32 tokens per workgroup, the model dimension split over the 4 wavefronts ---------------
+template <typename T>
+__global__ __launch_bounds__(256) void gate_fwd_kernel(float* __restrict__ logits, const T* __restrict__ x,
+                                                       const float* __restrict__ wg, int num_tokens, int d, int E) {
+    __shared__ float part[4][16][64];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 31, h = lane >> 5;
+    const int t0 = blockIdx.x * GT;
+    const int pieces = d >> 3;                       // 8 contraction indices per piece
+    const int chunks = (pieces + 1) >> 1;            // a chunk = one piece per half-wavefront
+    const int c0 = (chunks * wave) >> 2, c1 = (chunks * (wave + 1)) >> 2;
+    const bool tok_ok = t0 + r < num_tokens;
+    const T* xrow = x + (size_t)(t0 + r) * d;
+    for (int e0 = 0; e0 < E; e0 += 32) {
+        const bool exp_ok = e0 + r < E;
+        const float* wrow = wg + (size_t)(e0 + r) * d;
+        f32x16 acc = zero16();
+#pragma unroll 2
+        for (int c = c0; c < c1; ++c) {
+            const int piece = 2 * c + h;
+            const bool ok = piece < pieces;
+            float xv[8], wv[8];
+            LoadN<T, 8>::run(xrow + piece * 8, ok && tok_ok, xv);
+            LoadN<float, 8>::run(wrow + piece * 8, ok && exp_ok, wv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[i], wv[i], acc, 0, 0, 0);
+        }
+        __syncthreads();   // the previous expert block's partial sums have been consumed
+#pragma unroll
+        for (int v = 0; v < 16; ++v) part[wave][v][lane] = acc[v];
+        __syncthreads();
+        // wavefront w finishes result registers 4w..4w+3: token row 8w + 4h + q, expert column r
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int v = 4 * wave + q;
+            const float sum = ((part[0][v][lane] + part[1][v][lane]) + part[2][v][lane]) + part[3][v][lane];
+            const int t = t0 + 8 * wave + 4 * h + q;
+            if (t < num_tokens && exp_ok) logits[(size_t)t * E + e0 + r] = sum;
+        }
+    }
+}
+
+// ---- dx: 32 tokens per workgroup, 128-column groups of the model dimension over the wavefronts ------
+template <typename T>
+__global__ __launch_bounds__(256) void gate_dx_kernel(T* __restrict__ dx, const float* __restrict__ dl,
+                                                      const float* __restrict__ wg, int num_tokens, int d, int E) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 31, h = lane >> 5;
+    const int t0 = blockIdx.x * GT;
+    const bool tok_ok = t0 + r < num_tokens;
+    const float* drow = dl + (size_t)(t0 + r) * E;
+    for (int g = wave; g * 128 < d; g += 4) {
+        const int col = g * 128 + 4 * r;
+        const bool col_ok = col < d;
+        f32x16 acc[4] = {zero16(), zero16(), zero16(), zero16()};
+        for (int e0 = 0; e0 < E; e0 += 32) {
+            // this lane's contraction indices: experts e0 + 16h + 0..15
+            float a[16];
+            if ((E & 3) == 0) {   // rows are 16-byte aligned: four float4 loads
+#pragma unroll
+                for (int i = 0; i < 16; i += 4) {
+                    const int e = e0 + 16 * h + i;
+                    const float4 v = (tok_ok && e < E) ? *reinterpret_cast<const float4*>(drow + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    a[i] = v.x; a[i + 1] = v.y; a[i + 2] = v.z; a[i + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int e = e0 + 16 * h + i;
+                    a[i] = (tok_ok && e < E) ? drow[e] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int e = e0 + 16 * h + i;
+                float b[4];
+                LoadN<float, 4>::run(wg + (size_t)e * d + col, col_ok && e < E, b);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[j], 0, 0, 0);
+            }
+        }
+        if (col_ok) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int t = t0 + 8 * (v >> 2) + 4 * h + (v & 3);
+                if (t < num_tokens) store4<T>(dx + (size_t)t * d + col, acc[0][v], acc[1][v], acc[2][v], acc[3][v]);
+            }
+        }
+    }
+}
+
+// ---- dwg: partial sums over DWG_TB tokens per workgroup, then a reduction in workgroup order ---------
+template <typename T>
+__global__ __launch_bounds__(256) void gate_dwg_kernel(float* __restrict__ part, const float* __restrict__ dl,
+                                                       const T* __restrict__ x, int num_tokens, int d, int E) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 31, h = lane >> 5;
+    const int t0 = blockIdx.x * DWG_TB;
+    const int e0 = blockIdx.y * 32;
+    const bool exp_ok = e0 + r < E;
+    float* out = part + (size_t)blockIdx.x * E * d;
+    for (int g = wave; g * 128 < d; g += 4) {
+        const int col = g * 128 + 4 * r;
+        const bool col_ok = col < d;
+        f32x16 acc[4] = {zero16(), zero16(), zero16(), zero16()};
+#pragma unroll 8
+        for (int i = 0; i < DWG_TB / 2; ++i) {
+            const int t = t0 + 2 * i + h;          // this lane's contraction index: one token
+            const bool ok = t < num_tokens;
+            const float a = (ok && exp_ok) ? dl[(size_t)t * E + e0 + r] : 0.f;
+            float b[4];
+            LoadN<T, 4>::run(x + (size_t)t * d + col, ok && col_ok, b);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b[j], acc[j], 0, 0, 0);
+        }
+        if (col_ok) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int e = e0 + 8 * (v >> 2) + 4 * h + (v & 3);
+                if (e < E) store4<float>(out + (size_t)e * d + col, acc[0][v], acc[1][v], acc[2][v], acc[3][v]);
+            }
+        }
+    }
+}
+
+// dwg = sum of the partial results, in a fixed order: a workgroup takes 16 float4 columns; each of its
+// 16 thread groups sums a contiguous range of the partials, then the 16 group sums are added in order.
+__global__ __launch_bounds__(256) void gate_dwg_reduce_kernel(float* __restrict__ dwg, const float* __restrict__ part,
+                                                              int nparts, long n4) {
+    __shared__ float4 sums[16][16];
+    const int c = threadIdx.x & 15, grp = threadIdx.x >> 4;
+    const long i = (long)blockIdx.x * 16 + c;
+    const int b0 = (int)((long)nparts * grp / 16), b1 = (int)((long)nparts * (grp + 1) / 16);
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < n4) {
+#pragma unroll 6
+        for (int b = b0; b < b1; ++b) {
+            const float4 v = reinterpret_cast<const float4*>(part)[(size_t)b * n4 + i];
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+    }
+    sums[grp][c] = s;
+    __syncthreads();
+    if (grp == 0 && i < n4) {
+        float4 t = sums[0][c];
+#pragma unroll
+        for (int g = 1; g < 16; ++g) { const float4 v = sums[g][c]; t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w; }
+        reinterpret_cast<float4*>(dwg)[i] = t;
+    }
+}
+
+template <typename T>
+int gate_backward_t(void* dx, float* dwg, const float* dl, const void* x, const float* wg, int T_, int d, int E, float* ws,
+                    hipStream_t st) {
+    if (dx) {
+        hipLaunchKernelGGL(gate_dx_kernel<T>, dim3(div_up(T_, GT)), dim3(256), 0, st, (T*)dx, dl, wg, T_, d, E);
+        HEXA_CHECK_LAUNCH("gate_dx");
+    }
+    if (dwg) {
+        const int nparts = div_up(T_, DWG_TB);
+        hipLaunchKernelGGL(gate_dwg_kernel<T>, dim3(nparts, div_up(E, 32)), dim3(256), 0, st, ws, dl, (const T*)x, T_, d, E);
+        HEXA_CHECK_LAUNCH("gate_dwg");
+        const long n4 = (long)E * d / 4;
+        hipLaunchKernelGGL(gate_dwg_reduce_kernel, dim3((unsigned)div_up(n4, 16)), dim3(256), 0, st, dwg, ws, nparts, n4);
+        HEXA_CHECK_LAUNCH("gate_dwg_reduce");
+    }
+    return HEXA_OK;
+}
+
+}  // namespace
+}  // namespace hexa
+
+using namespace hexa;
+
+extern "C" int hexa_gate_logits(float* logits, const void* x, const float* wg, int T, int d, int E, int x_dt,
+                                void* stream) {
+    if (T < 0 || d < 1 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_logits: bad sizes T=%d d=%d E=%d", T, d, E);
+    if (T > 0 && (!logits || !x || !wg)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_logits: null pointer");
+    if (d % 8) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_gate_logits: model dim must be a multiple of 8 (got %d)", d);
+    if (T == 0) return HEXA_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid(div_up(T, GT)), block(256);
+    if (x_dt == HEXA_F32) hipLaunchKernelGGL(gate_fwd_kernel<float>, grid, block, 0, st, logits, (const float*)x, wg, T, d, E);
+    else if (x_dt == HEXA_BF16) hipLaunchKernelGGL(gate_fwd_kernel<__bf16>, grid, block, 0, st, logits, (const __bf16*)x, wg, T, d, E);
+    else if (x_dt == HEXA_F16) hipLaunchKernelGGL(gate_fwd_kernel<_Float16>, grid, block, 0, st, logits, (const _Float16*)x, wg, T, d, E);
+    else HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_logits: unknown element type");
+    HEXA_CHECK_LAUNCH("gate_fwd");
+    return HEXA_OK;
+}
+
+extern "C" int hexa_gate_ws_floats(int T, int d, int E, int64_t* out) {
+    if (!out || T < 0 || d < 1 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_ws_floats: bad arguments");
+    *out = (int64_t)(T > 0 ? div_up(T, DWG_TB) : 1) * E * d;
+    return HEXA_OK;
+}
+
+extern "C" int hexa_gate_backward(void* dx, float* dwg, const float* dlogits, const void* x, const float* wg, int T,
+                                  int d, int E, int x_dt, float* ws, void* stream) {
+    if (T < 0 || d < 1 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_backward: bad sizes T=%d d=%d E=%d", T, d, E);
+    if (d % 8) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_gate_backward: model dim must be a multiple of 8 (got %d)", d);
+    if (!dx && !dwg) return HEXA_OK;
+    if (T > 0 && (!dlogits || !wg || (dwg && (!x || !ws)))) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_backward: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    if (T == 0) {   // no tokens: dwg = 0 (a reduction over zero partial sums)
+        if (dwg) {
+            const long n4 = (long)E * d / 4;
+            hipLaunchKernelGGL(gate_dwg_reduce_kernel, dim3((unsigned)div_up(n4, 16)), dim3(256), 0, st, dwg, dwg, 0, n4);
+            HEXA_CHECK_LAUNCH("gate_dwg_reduce");
+        }
+        return HEXA_OK;
+    }
+    if (x_dt == HEXA_F32) return gate_backward_t<float>(dx, dwg, dlogits, x, wg, T, d, E, ws, st);
+    if (x_dt == HEXA_BF16) return gate_backward_t<__bf16>(dx, dwg, dlogits, x, wg, T, d, E, ws, st);
+    if (x_dt == HEXA_F16) return gate_backward_t<_Float16>(dx, dwg, dlogits, x, wg, T, d, E, ws, st);
+    HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_backward: unknown element type");
+}

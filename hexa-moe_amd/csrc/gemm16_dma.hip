@@ -32,17 +32,40 @@ namespace {
 
 template <typename TC, bool W_IN_OUT, bool OUT32, typename C>
 __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
-    constexpr int BM = C::BM, BN = C::BN, STAGES = C::STAGES, NW = C::NW;
+    constexpr int BM = C::BM, BN = C::BN, STAGES = C::STAGES, NW = C::NW, BK = C::BKC;
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     int* sTok = reinterpret_cast<int*>(smem + C::STAGE_AREA);
 
-    const long logical = logical_tile(p.group);
-    if (logical >= p.total) return;
-    const int nt = (int)(logical % p.ntn);
-    const int mtg = (int)(logical / p.ntn);
-    const int s = p.slot_begin + mtg / p.mt_ub;
-    const int mt = mtg % p.mt_ub;
-    if (mt >= p.tile_count[s]) return;
+    int nt, s, mt;
+    if (p.group > 0) {
+        const long logical = logical_tile(p.group);
+        if (logical >= p.total) return;
+        nt = (int)(logical % p.ntn);
+        const int mtg = (int)(logical / p.ntn);
+        s = p.slot_begin + mtg / p.mt_ub;
+        mt = mtg % p.mt_ub;
+        if (mt >= p.tile_count[s]) return;
+    } else {
+        // Every XCD (workgroup ids go round-robin over the 8 of them) walks one contiguous eighth of
+        // the list of VALID tiles, column tiles fastest: an expert's weights are then fetched into
+        // one L2 (two at a boundary) per slot instead of into all eight.
+        int cum[9];
+        cum[0] = 0;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) cum[q + 1] = cum[q] + (q < p.nslots ? min(p.tile_count[p.slot_begin + q], p.mt_ub) : 0);
+        const int valid = cum[8] * p.ntn;
+        const int per = (valid + 7) >> 3;
+        const int xcd = blockIdx.x & 7, loc = blockIdx.x >> 3;
+        const int logical = xcd * per + loc;
+        if (loc >= per || logical >= valid) return;
+        const int mtg = logical / p.ntn;
+        nt = logical - mtg * p.ntn;
+        int sl = 0;
+#pragma unroll
+        for (int q = 1; q < 8; ++q) sl += (mtg >= cum[q] && q < p.nslots) ? 1 : 0;
+        s = p.slot_begin + sl;
+        mt = mtg - cum[sl];
+    }
     const int4 info = p.tile_info[(size_t)s * p.mt_ub + mt];
     const int e = info.x, row_start = info.y, rows = info.z;
     const int n0 = nt * BN;
@@ -61,7 +84,7 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
 #pragma unroll
     for (int i = 0; i < C::R_CPW; ++i) {   // token rows, KC
         int row, kc;
-        kc_lane(wave + NW * i, lane, row, kc);
+        kc_lane<BK>(wave + NW * i, lane, row, kc);
         const int tok = sTok[row];
         const bool ok = tok >= 0;
         srcR[i] = ok ? reinterpret_cast<const char*>(p.x) + (((size_t)p.x_slot_rows * s + tok) * K + kc * 8) * 2 : zero;
@@ -78,7 +101,7 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
             stepF[i] = ok ? BK * N * 2 : 0;
         } else {         // w[e][n][k], KC
             int row, kc;
-            kc_lane(wave + NW * i, lane, row, kc);
+            kc_lane<BK>(wave + NW * i, lane, row, kc);
             const int n = n0 + row;
             const bool ok = n < N;
             srcF[i] = ok ? reinterpret_cast<const char*>(p.w) + (((size_t)e * N + n) * K + kc * 8) * 2 : zero;
@@ -177,15 +200,13 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
         }
         if (!OUT32) {
             __syncthreads();
-            constexpr int LPR = BN / 8;             // lanes per row
-            constexpr int RPI = C::NT / LPR;        // rows per iteration
-            const int c = tid % LPR, n = n0 + c * 8;
-            if (n < N) {
+            constexpr int LPR = BN / 8;             // 16-byte pieces per row
+            {
 #pragma unroll 4
-                for (int it = 0; it < PR / RPI; ++it) {
-                    const int rl = it * RPI + tid / LPR;
+                for (int idx = tid; idx < PR * LPR; idx += C::NT) {
+                    const int rl = idx / LPR, c = idx - rl * LPR, n = n0 + c * 8;
                     const int tok = sTok[pass * PR + rl];
-                    if (tok < 0) continue;
+                    if (tok < 0 || n >= N) continue;
                     const size_t off = (out_base + tok) * N + n;
                     uint4 val = *reinterpret_cast<const uint4*>(smem + rl * CP + c * 16);
                     uint4* dst = reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(outp) + off);
@@ -230,6 +251,12 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
     }
 }
 
+// integer tuning knob from the environment (read on every call: testing aid only)
+static int env_int(const char* name, int dflt) {
+    const char* s = getenv(name);
+    return s ? atoi(s) : dflt;
+}
+
 template <typename TC, bool IO, bool OUT32, typename C>
 int launch_esmm_dma_t(EsmmK& p, int grid, hipStream_t st) {
     auto kernel = esmm16_dma_kernel<TC, IO, OUT32, C>;
@@ -266,7 +293,12 @@ struct Cursor {   // walks the expert's token list in 32-token steps, slot after
 };
 
 // fp32 result rows staged per pass, and the LDS area that holds both the stages and that staging
-template <typename C> constexpr int estmm_pass_rows() { return C::BN <= 128 ? 128 : 64; }
+template <typename C> constexpr int estmm_pass_rows() {
+    // the largest multiple-of-32 divisor of BM whose staged fp32 rows fit in the stage buffers
+    for (int rows = C::BM; rows > 32; rows /= 2)
+        if (rows * (C::BN + 4) * 4 <= C::STAGE_AREA) return rows;
+    return 32;
+}
 template <typename C> constexpr int estmm_stage_area() {
     constexpr int staged = estmm_pass_rows<C>() * (C::BN + 4) * 4;
     return C::STAGE_AREA > staged ? C::STAGE_AREA : staged;
@@ -275,6 +307,7 @@ template <typename C> constexpr int estmm_stage_area() {
 template <typename TC, bool OUT32, typename C>
 __global__ __launch_bounds__(C::NT, C::MINW) void estmm16_dma_kernel(EstmmK p) {
     constexpr int BM = C::BM, BN = C::BN, STAGES = C::STAGES, NW = C::NW;
+    static_assert(C::BKC == 32, "token ids travel 32 per step");
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     int* sIds = reinterpret_cast<int*>(smem + estmm_stage_area<C>());       // [TOK_RING][32]
     __shared__ int sBeg[MAX_SLOTS], sEnd[MAX_SLOTS];
@@ -421,8 +454,7 @@ __global__ __launch_bounds__(C::NT, C::MINW) void estmm16_dma_kernel(EstmmK p) {
     float* sC = reinterpret_cast<float*>(smem);
     constexpr int CPF = BN + 4;
     constexpr int PRF = estmm_pass_rows<C>();
-    constexpr int LPRF = BN / 4;              // lanes per row
-    constexpr int RPI = C::NT / LPRF;         // rows stored per iteration
+    constexpr int LPRF = BN / 4;              // 16-byte (fp32) pieces per row
     constexpr int RW = 32 * C::RB, FW = 32 * C::FB;
 #pragma unroll
     for (int h = 0; h < BM / PRF; ++h) {
@@ -443,13 +475,12 @@ __global__ __launch_bounds__(C::NT, C::MINW) void estmm16_dma_kernel(EstmmK p) {
             }
         }
         __syncthreads();
-        const int c = tid % LPRF, n = n0 + c * 4;
-        if (n < N) {
+        {
 #pragma unroll 4
-            for (int it = 0; it < PRF / RPI; ++it) {
-                const int ml = it * RPI + tid / LPRF;
+            for (int idx = tid; idx < PRF * LPRF; idx += C::NT) {
+                const int ml = idx / LPRF, c = idx - ml * LPRF, n = n0 + c * 4;
                 const int m = m0 + h * PRF + ml;
-                if (m >= M) break;
+                if (m >= M || n >= N) continue;
                 float4 v = *reinterpret_cast<const float4*>(sC + ml * CPF + c * 4);
                 const size_t off = ((size_t)e * M + m) * N + n;
                 if (OUT32) {
@@ -490,7 +521,7 @@ int launch_estmm_dma_c(const EstmmArgs& a, hipStream_t st) {
     p.p_slot_rows = a.p_per_slot ? a.r.T : 0;
     p.q_slot_rows = a.q_per_slot ? a.r.T : 0;
     p.accumulate = a.accumulate;
-    p.group = p.ntn;
+    p.group = p.ntn * env_int("HEXA_ESTMM_GROUP", 1);
     p.total = (long)a.r.E * p.mtn * p.ntn;
     if (p.total == 0) return HEXA_OK;
     const int grid = round_up(p.total, 8 * p.group);
@@ -512,7 +543,7 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
     p.x_slot_rows = a.x_per_slot ? a.r.T : 0;
     p.out_slot_rows = a.out_per_slot ? a.r.T : 0;
     p.bias_dt = a.bias_dt; p.out_dt = a.out_dt; p.act = a.act;
-    p.group = p.ntn * (large ? 2 : 4);
+    p.group = p.ntn * env_int("HEXA_ESMM_GROUP", large ? 2 : 4);
     // Summing the slots into one result: with scratch, every slot runs in ONE launch (slot 0 into
     // `out`, the others into the scratch) and a reduction adds them in slot order; without it, one
     // launch per slot, each adding into `out`.
@@ -525,7 +556,9 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
         p.accumulate = (a.accumulate || l > 0) ? 1 : 0;
         p.total = (long)p.nslots * p.mt_ub * p.ntn;
         if (p.total == 0) continue;
-        const int grid = round_up(p.total, 8 * p.group);
+        const bool contiguous = p.nslots <= 8 && env_int("HEXA_ESMM_MAP", 0) == 1;
+        const int grid = round_up(p.total, contiguous ? 8 : 8 * p.group);
+        if (contiguous) p.group = 0;
         const bool io = a.w_layout == HEXA_W_IN_OUT;
         const bool o32 = a.out_dt == HEXA_F32;
         const int rc = a.x_dt == HEXA_BF16 ? launch_esmm_dma_d<__bf16, C>(p, grid, io, o32, st)
@@ -536,23 +569,25 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
     return HEXA_OK;
 }
 
-// 0: automatic; 1: 128x128; 2: 256x128 (8 wavefronts); 3: 256x128 (4 wavefronts); 4: 256x256
-// (HEXA_MOE_TILE, testing aid, read once)
+// HEXA_MOE_TILE (testing aid, read once): 0 automatic; 1 128x128; 2 256x128 (8 wavefronts); 3 256x128
+// (4 wavefronts); 4..6 256x256 (4 / 8 / 16 wavefronts); 7 128x384; 8, 9 128x128 with 4 / 3 workgroups
+// per CU; 10, 11 128x128 / 256x128 with 64 contraction indices per stage (ESMM only)
 int forced_tile() {
     static const int v = [] { const char* s = getenv("HEXA_MOE_TILE"); return s ? atoi(s) : 0; }();
     return v;
 }
 
-int pick_esmm_tile(long rows, int cols) {
+int pick_esmm_tile(long rows, int cols, int in_dim) {
     const int f = forced_tile();
     if (f) return f;
-    return rows / 256 * div_up(cols, 128) >= 512 ? 2 : 1;
+    if (rows / 256 * div_up(cols, 128) >= 512) return 2;      // enough 256-row tiles to fill the chip
+    return (in_dim % 64) == 0 ? 10 : 1;                       // whole 128-byte lines per row and stage when possible
 }
 
 }  // namespace
 
 bool esmm16_dma_supported(const EsmmArgs& a) {
-    return a.w_dt == a.x_dt && (a.in_dim % BK) == 0 && (a.out_dim % 8) == 0 &&
+    return a.w_dt == a.x_dt && (a.in_dim % 32) == 0 && (a.out_dim % 8) == 0 &&
            (a.out_dt == a.x_dt || a.out_dt == HEXA_F32);
 }
 
@@ -561,12 +596,18 @@ bool estmm16_dma_supported(const EstmmArgs& a) {
 }
 
 int launch_estmm16_dma(const EstmmArgs& a, hipStream_t st) {
+    // a result up to 384 wide is spanned by ONE tile: the tall operand (m_dim columns of every token
+    // row) is then fetched once instead of once per column tile
+    // (measured: not a gain while the longest expert's token list bounds the kernel, so only on request)
+    if (forced_tile() == 7) return launch_estmm_dma_c<CfgW>(a, st);
     switch (forced_tile()) {
         case 2: return launch_estmm_dma_c<CfgL>(a, st);
         case 3: return launch_estmm_dma_c<CfgM>(a, st);
         case 4: return launch_estmm_dma_c<CfgX>(a, st);
         case 5: return launch_estmm_dma_c<CfgX8>(a, st);
         case 6: return launch_estmm_dma_c<CfgX16>(a, st);
+        case 8: return launch_estmm_dma_c<CfgS2>(a, st);
+        case 9: return launch_estmm_dma_c<CfgS3>(a, st);
         default: return launch_estmm_dma_c<CfgS>(a, st);
     }
 }
@@ -580,12 +621,17 @@ static bool persist_enabled() {
 
 int launch_esmm16_dma(const EsmmArgs& a, hipStream_t st) {
     if (persist_enabled() && esmm16_persist_supported(a)) return launch_esmm16_persist(a, forced_tile(), st);
-    switch (pick_esmm_tile((long)a.r.T * a.r.k, a.out_dim)) {
+    if (forced_tile() == 7) return launch_esmm_dma_c<CfgW>(a, false, st);
+    switch (pick_esmm_tile((long)a.r.T * a.r.k, a.out_dim, a.in_dim)) {
         case 2: return launch_esmm_dma_c<CfgL>(a, true, st);
         case 3: return launch_esmm_dma_c<CfgM>(a, true, st);
         case 4: return launch_esmm_dma_c<CfgX>(a, true, st);
         case 5: return launch_esmm_dma_c<CfgX8>(a, true, st);
         case 6: return launch_esmm_dma_c<CfgX16>(a, true, st);
+        case 8: return launch_esmm_dma_c<CfgS2>(a, false, st);
+        case 10: return (a.in_dim % 64) ? launch_esmm_dma_c<CfgS>(a, false, st) : launch_esmm_dma_c<CfgS64>(a, false, st);
+        case 11: return (a.in_dim % 64) ? launch_esmm_dma_c<CfgL>(a, true, st) : launch_esmm_dma_c<CfgL64>(a, true, st);
+        case 9: return launch_esmm_dma_c<CfgS3>(a, false, st);
         default: return launch_esmm_dma_c<CfgS>(a, false, st);
     }
 }

@@ -1,5 +1,5 @@
-// Routing front end for gfx950: gate projection, softmax + top-k + GShard auxiliary loss, and the
-// loss's backward through the softmax.  These are small HBM-/latency-bound kernels that replace a
+// Routing front end for gfx950: softmax + top-k + GShard auxiliary loss, and the loss's backward
+// through the softmax (the gate projection itself is in gate.hip).  These are small HBM-/latency-bound kernels that replace a
 // dozen framework launches per MoE depth (fp32 cast, a skinny fp32 GEMM, softmax, top-k select + sort,
 // one-hot scatter, reductions).
 //
@@ -10,101 +10,6 @@
 
 namespace hexa {
 namespace {
-
-// ---- gate projection: logits[t][e] = sum_d x[t][d] * wg[e][d], fp32 accumulation ---------------------
-// 64 tokens per workgroup, one token per lane.  The model dimension is processed in chunks of 256:
-// the chunk of the 64 token rows and of 32 gate rows is staged in LDS with coalesced 16-byte loads;
-// each of the 4 wavefronts takes a quarter of the chunk, reads its token's pieces from LDS and the
-// gate row pieces as LDS broadcasts (one address for the whole wavefront), and the four partial sums
-// are folded through LDS in a fixed order.
-constexpr int GATE_EB = 32;    // experts per pass
-constexpr int GATE_DC = 256;   // model-dim chunk
-constexpr int GATE_XP = GATE_DC + 8;    // pitch of a staged token row, in elements (16 B of padding)
-constexpr int GATE_WP = GATE_DC + 4;    // pitch of a staged gate row, in floats
-
-template <typename T> struct Row8;   // 8 consecutive elements as floats
-template <> struct Row8<float> {
-    static __device__ __forceinline__ void load(const float* p, float (&v)[8]) {
-        const float4 a = reinterpret_cast<const float4*>(p)[0], b = reinterpret_cast<const float4*>(p)[1];
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-    }
-};
-template <typename T16> struct Row8 {
-    static __device__ __forceinline__ void load(const T16* p, float (&v)[8]) {
-        union { uint4 u; T16 e[8]; } r;
-        r.u = *reinterpret_cast<const uint4*>(p);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = (float)r.e[i];
-    }
-};
-
-template <typename T> constexpr int gate_smem_bytes() {
-    return 64 * GATE_XP * (int)sizeof(T) + GATE_EB * GATE_WP * 4 + 3 * 64 * (GATE_EB + 1) * 4;
-}
-
-template <typename T>
-__global__ __launch_bounds__(256) void gate_logits_kernel(float* __restrict__ logits, const T* __restrict__ x,
-                                                          const float* __restrict__ wg, int num_tokens, int d,
-                                                          int E) {
-    extern __shared__ __attribute__((aligned(16))) char gsm[];
-    T* sX = reinterpret_cast<T*>(gsm);
-    float* sW = reinterpret_cast<float*>(gsm + 64 * GATE_XP * sizeof(T));
-    float (*part)[64][GATE_EB + 1] = reinterpret_cast<float (*)[64][GATE_EB + 1]>(sW + GATE_EB * GATE_WP);
-    constexpr int VX = 16 / (int)sizeof(T);   // elements per 16-byte piece of a token row
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int t0 = blockIdx.x * 64;
-    const int t = t0 + lane;
-    for (int e0 = 0; e0 < E; e0 += GATE_EB) {
-        float acc[GATE_EB];
-#pragma unroll
-        for (int e = 0; e < GATE_EB; ++e) acc[e] = 0.f;
-        for (int d0 = 0; d0 < d; d0 += GATE_DC) {
-            const int dc = min(GATE_DC, d - d0);          // multiple of 8
-            __syncthreads();                               // previous chunk fully consumed
-            for (int i = tid; i < 64 * (dc / VX); i += 256) {
-                const int r = i / (dc / VX), c = i - r * (dc / VX);
-                uint4 v = make_uint4(0u, 0u, 0u, 0u);
-                if (t0 + r < num_tokens) v = *reinterpret_cast<const uint4*>(x + (size_t)(t0 + r) * d + d0 + c * VX);
-                *reinterpret_cast<uint4*>(sX + r * GATE_XP + c * VX) = v;
-            }
-            for (int i = tid; i < GATE_EB * (dc / 4); i += 256) {
-                const int r = i / (dc / 4), c = i - r * (dc / 4);
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (e0 + r < E) v = *reinterpret_cast<const float4*>(wg + (size_t)(e0 + r) * d + d0 + c * 4);
-                *reinterpret_cast<float4*>(sW + r * GATE_WP + c * 4) = v;
-            }
-            __syncthreads();
-            const int pieces = dc >> 3;
-            const int p0 = (pieces * wave) >> 2, p1 = (pieces * (wave + 1)) >> 2;
-            for (int pc = p0; pc < p1; ++pc) {
-                float xv[8];
-                Row8<T>::load(sX + lane * GATE_XP + pc * 8, xv);
-#pragma unroll
-                for (int e = 0; e < GATE_EB; ++e) {
-                    const float4 w0 = *reinterpret_cast<const float4*>(sW + e * GATE_WP + pc * 8);      // broadcast
-                    const float4 w1 = *reinterpret_cast<const float4*>(sW + e * GATE_WP + pc * 8 + 4);
-                    float a = acc[e];
-                    a = fmaf(xv[0], w0.x, a); a = fmaf(xv[1], w0.y, a); a = fmaf(xv[2], w0.z, a); a = fmaf(xv[3], w0.w, a);
-                    a = fmaf(xv[4], w1.x, a); a = fmaf(xv[5], w1.y, a); a = fmaf(xv[6], w1.z, a); a = fmaf(xv[7], w1.w, a);
-                    acc[e] = a;
-                }
-            }
-        }
-        if (wave > 0) {
-#pragma unroll
-            for (int e = 0; e < GATE_EB; ++e) part[wave - 1][lane][e] = acc[e];
-        }
-        __syncthreads();
-        if (wave == 0 && t < num_tokens) {
-#pragma unroll
-            for (int e = 0; e < GATE_EB; ++e) {
-                if (e0 + e < E)
-                    logits[(size_t)t * E + e0 + e] = ((acc[e] + part[0][lane][e]) + part[1][lane][e]) + part[2][lane][e];
-            }
-        }
-    }
-}
 
 // ---- softmax + top-k + per-workgroup loss partials ----------------------------------------------------
 // One token per lane, three passes over its logits row (max, sum of exp, scores + selection); the row
@@ -245,40 +150,11 @@ __global__ __launch_bounds__(ROUTER_TB) void router_bwd_kernel(float* __restrict
     }
 }
 
-template <typename T>
-int launch_gate(dim3 grid, dim3 block, hipStream_t st, float* logits, const void* x, const float* wg, int num_tokens,
-                int d, int E) {
-    static bool attr_done = false;
-    constexpr int bytes = gate_smem_bytes<T>();
-    if (!attr_done) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(gate_logits_kernel<T>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
-            HEXA_FAIL(HEXA_ERR_LAUNCH, "hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d) failed", bytes);
-        attr_done = true;
-    }
-    hipLaunchKernelGGL(gate_logits_kernel<T>, grid, block, bytes, st, logits, (const T*)x, wg, num_tokens, d, E);
-    HEXA_CHECK_LAUNCH("gate_logits");
-    return HEXA_OK;
-}
 
 }  // namespace
 }  // namespace hexa
 
 using namespace hexa;
-
-extern "C" int hexa_gate_logits(float* logits, const void* x, const float* wg, int T, int d, int E, int x_dt,
-                                void* stream) {
-    if (T < 0 || d < 1 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_logits: bad sizes T=%d d=%d E=%d", T, d, E);
-    if (T > 0 && (!logits || !x || !wg)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_logits: null pointer");
-    if (d % 8) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_gate_logits: model dim must be a multiple of 8 (got %d)", d);
-    if (T == 0) return HEXA_OK;
-    hipStream_t st = (hipStream_t)stream;
-    const dim3 grid(div_up(T, 64)), block(256);
-    if (x_dt == HEXA_F32) return launch_gate<float>(grid, block, st, logits, x, wg, T, d, E);
-    if (x_dt == HEXA_BF16) return launch_gate<__bf16>(grid, block, st, logits, x, wg, T, d, E);
-    if (x_dt == HEXA_F16) return launch_gate<_Float16>(grid, block, st, logits, x, wg, T, d, E);
-    HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_logits: unknown element type");
-}
 
 extern "C" int hexa_router_ws_floats(int T, int E, int64_t* out) {
     if (!out || T < 0 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_router_ws_floats: bad arguments");

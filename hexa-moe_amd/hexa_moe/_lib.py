@@ -40,6 +40,8 @@ SIGNATURES = {
     "hexa_fused_grad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "hexa_gelu_bwd": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),
     "hexa_gate_logits": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "hexa_gate_ws_floats": (_i, [_i, _i, _i, ctypes.POINTER(_i64)]),
+    "hexa_gate_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "hexa_router_ws_floats": (_i, [_i, _i, ctypes.POINTER(_i64)]),
     "hexa_router_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float, _i, _i, _i, _vp, _vp]),
     "hexa_router_backward": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),

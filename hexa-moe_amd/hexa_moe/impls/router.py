@@ -21,11 +21,9 @@ class GateProjection(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dlogits):
         x, wg = ctx.saved_tensors
-        dx = dwg = None
-        if ctx.needs_input_grad[0]:
-            dx = (dlogits @ wg.float()).to(x.dtype)
-        if ctx.needs_input_grad[1]:
-            dwg = (dlogits.t() @ x.float()).to(wg.dtype)
+        dx, dwg = ops.gate_backward(dlogits, x, wg.float(), ctx.needs_input_grad[0], ctx.needs_input_grad[1])
+        if dwg is not None:
+            dwg = dwg.to(wg.dtype)
         return dx, dwg
 
 

@@ -255,6 +255,30 @@ def gate_logits(x, wg):
     return logits
 
 
+def gate_backward(dlogits, x, wg, need_dx=True, need_dwg=True):
+    """Backward of gate_logits: (dx [T, d] in x's type or None, dwg [E, d] fp32 or None)."""
+    import ctypes
+    _dev(dlogits, x, wg)
+    dlogits = dlogits.contiguous()
+    x = x.contiguous()
+    wg = wg.contiguous()
+    assert dlogits.dtype == torch.float32 and wg.dtype == torch.float32
+    T, d = x.shape
+    E = wg.shape[0]
+    assert dlogits.shape == (T, E) and wg.shape == (E, d)
+    dx = torch.empty_like(x) if need_dx else None
+    dwg = ws = None
+    if need_dwg:
+        n = ctypes.c_int64()
+        _lib.check(_lib.load().hexa_gate_ws_floats(T, d, E, ctypes.byref(n)), "hexa_gate_ws_floats")
+        ws = torch.empty(int(n.value), dtype=torch.float32, device=x.device)
+        dwg = torch.empty(E, d, dtype=torch.float32, device=x.device)
+    rc = _call("gate_backward", _lib.load().hexa_gate_backward, _ptr(dx), _ptr(dwg), _ptr(dlogits), _ptr(x), _ptr(wg),
+               T, d, E, _dt(x), _ptr(ws), _stream())
+    _lib.check(rc, "hexa_gate_backward")
+    return dx, dwg
+
+
 def router_forward(logits, top_k, noise=None, noise_scale=0.0):
     """softmax + top-k + GShard loss.  Returns scores [T,E] fp32, idx [T,k] int32, me [E], ce [E], l_aux []."""
     import ctypes

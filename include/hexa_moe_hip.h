@@ -166,6 +166,15 @@ int hexa_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt,
 int hexa_gate_logits(float* logits, const void* x, const float* wg, int num_tokens, int model_dim,
                      int num_experts, int x_dt, void* stream);
 
+/* Backward of the gate projection: dx[t][c] = sum_e dlogits[t][e]*wg[e][c] (type of x; NULL to skip) and
+ * dwg[e][c] = sum_t dlogits[t][e]*x[t][c] (fp32; NULL to skip), both with fp32 products and sums.  dwg is
+ * reduced over per-workgroup partial sums in a fixed order (deterministic); `ws` holds them and must have
+ * hexa_gate_ws_floats() floats.  Replaces what autograd derives from gates/top.py:17-19 (two skinny fp32
+ * GEMMs and the casts around them). */
+int hexa_gate_ws_floats(int num_tokens, int model_dim, int num_experts, int64_t* out);
+int hexa_gate_backward(void* dx, float* dwg, const float* dlogits, const void* x, const float* wg, int num_tokens,
+                       int model_dim, int num_experts, int x_dt, float* ws, void* stream);
+
 /* softmax(logits + noise_scale*noise) -> scores [T][E]; top-k expert ids idx [T][k] (int32, descending
  * score, ties to the lower id); me[e] = sum_t scores, ce[e] = (E/T)*#{t: top-1 = e}; l_aux =
  * sum_e me*ce / T (the GShard loss).  noise may be NULL.  ws: hexa_router_ws_floats() floats.

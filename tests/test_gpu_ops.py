@@ -27,6 +27,8 @@ SHAPES = [
     (700, 200, 72, 4, 1, "one"),
     (2048, 128, 512, 8, 1, None),
     (1500, 264, 392, 16, 2, "zipf"),
+    (1100, 512, 384, 8, 2, None),     # a 384-wide result: one tile spans it
+    (900, 96, 328, 5, 2, "zipf"),
 ]
 
 

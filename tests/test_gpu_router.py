@@ -25,6 +25,29 @@ def test_gate_logits(dev, dtype, T, d, E):
     assert_close(got, want, 2e-6, "gate logits")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,d,E", [(1000, 384, 32), (77, 128, 8), (300, 264, 70), (18432, 384, 32), (33, 8, 3)])
+def test_gate_backward(dev, dtype, T, d, E):
+    """dx = dlogits . wg (in x's type) and dwg = dlogits^T . x (fp32), fp32 products and sums."""
+    from hexa_moe import ops
+    g = gen(T + E + d)
+    x = torch.randn(T, d, generator=g).to(dtype)
+    wg = torch.randn(E, d, generator=g) / d ** 0.5
+    dl = torch.randn(T, E, generator=g)
+    want_dx = dl.double() @ wg.double()
+    want_dwg = dl.double().t() @ x.double()
+    dx, dwg = ops.gate_backward(dl.to(dev), x.to(dev), wg.to(dev))
+    torch.cuda.synchronize()
+    assert dx.dtype == dtype and dwg.dtype == torch.float32
+    assert_close(dwg, want_dwg, 2e-6, "gate dwg")
+    assert_close(dx, want_dx, 2e-6 if dtype == torch.float32 else 2e-2, "gate dx")
+    dx_only, none = ops.gate_backward(dl.to(dev), x.to(dev), wg.to(dev), need_dwg=False)
+    assert none is None and torch.equal(dx_only, dx)
+    # two runs give the same bits (fixed reduction order)
+    _, dwg2 = ops.gate_backward(dl.to(dev), x.to(dev), wg.to(dev), need_dx=False)
+    assert torch.equal(dwg, dwg2)
+
+
 @pytest.mark.parametrize("T,E,k", [(1000, 32, 2), (18432, 32, 2), (2048, 8, 1), (513, 70, 3), (64, 4, 4)])
 @pytest.mark.parametrize("with_noise", [False, True])
 def test_router_forward_and_backward(dev, T, E, k, with_noise):

@@ -18,54 +18,119 @@ constexpr int MAX_TOPK = 8;
 
 constexpr int ROUTER_TB = 64;   // tokens (= lanes) per workgroup of the softmax/top-k kernel
 
+constexpr int ROUTER_LDS_E = 240;   // up to this many experts the 64 x E tile is staged in LDS
+constexpr int ROUTER_P = ROUTER_TB + 1;   // pitch of one expert's 64 values
+
+// insertion of (cv, ci) into a descending list of k entries; strict '>' keeps the lower index on ties
+__device__ __forceinline__ void topk_insert(float (&best_v)[MAX_TOPK], int (&best_i)[MAX_TOPK], int k, float cv, int ci) {
+#pragma unroll
+    for (int j = 0; j < MAX_TOPK; ++j) {
+        if (j < k && cv > best_v[j]) {
+            const float tv = best_v[j]; const int ti = best_i[j];
+            best_v[j] = cv; best_i[j] = ci; cv = tv; ci = ti;
+        }
+    }
+}
+
+// STAGED: the workgroup's 64 x E tile of (logits + noise) is brought into LDS with coalesced loads,
+// stored expert-major (conflict-free for one token per lane), turned into scores in place, summed per
+// expert and written back coalesced.  Otherwise every lane walks its own row in global memory (three
+// passes, L1-resident) and the per-expert sums are wavefront reductions.
+template <bool STAGED>
 __global__ __launch_bounds__(ROUTER_TB) void router_fwd_kernel(float* __restrict__ scores, int32_t* __restrict__ idx,
                                                          float* __restrict__ part_me, float* __restrict__ part_cnt,
                                                          const float* __restrict__ logits,
                                                          const float* __restrict__ noise, float noise_scale,
                                                          int num_tokens, int E, int k) {
-    extern __shared__ float sh[];          // me[E] column sums of the wavefront, then cnt[E]
+    extern __shared__ float sh[];          // me[E] column sums of the wavefront, cnt[E], then the tile
     float* s_me = sh;
     float* s_cnt = sh + E;
+    float* tile = sh + 2 * E;              // [E][ROUTER_P]
     for (int i = threadIdx.x; i < 2 * E; i += blockDim.x) sh[i] = 0.f;
-    __syncthreads();
     const int lane = threadIdx.x;
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    const int t0 = blockIdx.x * ROUTER_TB;
+    const int t = t0 + lane;
     const bool ok = t < num_tokens;
-    const float* lr = logits + (size_t)(ok ? t : 0) * E;
-    const float* nr = noise ? noise + (size_t)(ok ? t : 0) * E : nullptr;
-    float mx = -INFINITY;
-    for (int e = 0; e < E; ++e) {
-        const float v = nr ? lr[e] + noise_scale * nr[e] : lr[e];
-        mx = fmaxf(mx, v);
+    const int rows = min(ROUTER_TB, num_tokens - t0);
+    // staging geometry: lpr lanes (a power of two >= E, at most 64) per token row
+    int lpr = 1;
+    while (lpr < E && lpr < ROUTER_TB) lpr <<= 1;
+    const int rpi = ROUTER_TB / lpr, sub_r = lane / lpr, sub_e = lane & (lpr - 1);
+    if (STAGED) {
+        // 8 row groups per trip, loads first: the global latency is paid once per trip, not per row
+        for (int e0 = 0; e0 < E; e0 += lpr) {
+            const int e = e0 + sub_e;
+            for (int r0 = 0; r0 < rows; r0 += 8 * rpi) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int r = r0 + u * rpi + sub_r;
+                    const bool in = r < rows && e < E;
+                    const size_t g = (size_t)(t0 + r) * E + e;
+                    v[u] = in ? logits[g] : 0.f;
+                    if (in && noise) v[u] += noise_scale * noise[g];
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int r = r0 + u * rpi + sub_r;
+                    if (r < rows && e < E) tile[e * ROUTER_P + r] = v[u];
+                }
+            }
+        }
     }
-    float sum = 0.f;
-    for (int e = 0; e < E; ++e) {
-        const float v = nr ? lr[e] + noise_scale * nr[e] : lr[e];
-        sum += expf(v - mx);
-    }
-    const float inv = 1.0f / sum;
+    __syncthreads();
     float best_v[MAX_TOPK];
     int best_i[MAX_TOPK];
 #pragma unroll
     for (int j = 0; j < MAX_TOPK; ++j) { best_v[j] = -INFINITY; best_i[j] = 0x7fffffff; }
-    for (int e = 0; e < E; ++e) {        // uniform trip count: every lane takes part in the reductions
-        const float v = nr ? lr[e] + noise_scale * nr[e] : lr[e];
-        const float sc = ok ? expf(v - mx) * inv : 0.f;
-        if (ok) scores[(size_t)t * E + e] = sc;
-        // insertion into the descending list; strict '>' keeps the lower index on ties
-        float cv = sc; int ci = e;
-#pragma unroll
-        for (int j = 0; j < MAX_TOPK; ++j) {
-            if (j < k && cv > best_v[j]) {
-                const float tv = best_v[j]; const int ti = best_i[j];
-                best_v[j] = cv; best_i[j] = ci; cv = tv; ci = ti;
+    if (STAGED) {
+        float* col = tile + lane;          // this token's values, ROUTER_P apart
+        float mx = -INFINITY;
+        if (ok) {
+#pragma unroll 8
+            for (int e = 0; e < E; ++e) mx = fmaxf(mx, col[e * ROUTER_P]);
+            float sum = 0.f;
+#pragma unroll 8
+            for (int e = 0; e < E; ++e) {
+                const float ex = expf(col[e * ROUTER_P] - mx);
+                col[e * ROUTER_P] = ex;
+                sum += ex;
             }
-        }
-        // column sum over the wavefront: xor butterfly, a fixed summation tree
-        float r = sc;
+            const float inv = 1.0f / sum;
+            float thresh = -INFINITY;      // k-th best so far
+#pragma unroll 4
+            for (int e = 0; e < E; ++e) {
+                const float sc = col[e * ROUTER_P] * inv;
+                col[e * ROUTER_P] = sc;
+                if (sc > thresh) {
+                    topk_insert(best_v, best_i, k, sc, e);
 #pragma unroll
-        for (int m = 32; m > 0; m >>= 1) r += __shfl_xor(r, m);
-        if (lane == 0) s_me[e] = r;
+                    for (int j = 0; j < MAX_TOPK; ++j)
+                        if (j == k - 1) thresh = best_v[j];
+                }
+            }
+        } else {
+            for (int e = 0; e < E; ++e) col[e * ROUTER_P] = 0.f;
+        }
+    } else {
+        const float* lr = logits + (size_t)(ok ? t : 0) * E;
+        const float* nr = noise ? noise + (size_t)(ok ? t : 0) * E : nullptr;
+        float mx = -INFINITY;
+        for (int e = 0; e < E; ++e) mx = fmaxf(mx, nr ? lr[e] + noise_scale * nr[e] : lr[e]);
+        float sum = 0.f;
+        for (int e = 0; e < E; ++e) sum += expf((nr ? lr[e] + noise_scale * nr[e] : lr[e]) - mx);
+        const float inv = 1.0f / sum;
+        for (int e = 0; e < E; ++e) {        // uniform trip count: every lane takes part in the reductions
+            const float v = nr ? lr[e] + noise_scale * nr[e] : lr[e];
+            const float sc = ok ? expf(v - mx) * inv : 0.f;
+            if (ok) scores[(size_t)t * E + e] = sc;
+            topk_insert(best_v, best_i, k, sc, e);
+            // column sum over the wavefront: xor butterfly, a fixed summation tree
+            float r = sc;
+#pragma unroll
+            for (int m = 32; m > 0; m >>= 1) r += __shfl_xor(r, m);
+            if (lane == 0) s_me[e] = r;
+        }
     }
     if (ok) {
 #pragma unroll
@@ -74,6 +139,24 @@ __global__ __launch_bounds__(ROUTER_TB) void router_fwd_kernel(float* __restrict
         atomicAdd(&s_cnt[best_i[0]], 1.0f);            // exact: at most 64 ones per counter
     }
     __syncthreads();
+    if (STAGED) {
+        // per-expert sums over the 64 tokens, in token order; then the scores leave coalesced
+        for (int e = lane; e < E; e += ROUTER_TB) {
+            float m = 0.f;
+#pragma unroll 16
+            for (int r = 0; r < ROUTER_TB; ++r) m += tile[e * ROUTER_P + r];
+            s_me[e] = m;
+        }
+        for (int e0 = 0; e0 < E; e0 += lpr) {
+            const int e = e0 + sub_e;
+#pragma unroll 8
+            for (int r0 = 0; r0 < rows; r0 += rpi) {
+                const int r = r0 + sub_r;
+                if (r < rows && e < E) scores[(size_t)(t0 + r) * E + e] = tile[e * ROUTER_P + r];
+            }
+        }
+        __syncthreads();
+    }
     for (int e = threadIdx.x; e < E; e += blockDim.x) {
         part_me[(size_t)blockIdx.x * E + e] = s_me[e];
         part_cnt[(size_t)blockIdx.x * E + e] = s_cnt[e];
@@ -85,17 +168,19 @@ __global__ __launch_bounds__(256) void router_loss_kernel(float* __restrict__ l_
                                                           float* __restrict__ ce, const float* __restrict__ part_me,
                                                           const float* __restrict__ part_cnt, int nblocks,
                                                           int num_tokens, int E) {
-    // per expert: 8 threads sum 8 contiguous ranges of the workgroup partials, then the 8 range sums
+    // per expert: nch threads sum nch contiguous ranges of the workgroup partials, then the range sums
     // are added in range order -- a fixed tree, independent of scheduling
-    extern __shared__ float sh[];          // [8][E] me, [8][E] cnt
+    extern __shared__ float sh[];          // [nch][E] me, [nch][E] cnt
+    const int nch = max(1, min(32, 8192 / E));
     float* s_m = sh;
-    float* s_c = sh + 8 * E;
+    float* s_c = sh + nch * E;
     __shared__ float red[256];
-    const int per = (nblocks + 7) / 8;
-    for (int i = threadIdx.x; i < 8 * E; i += 256) {
+    const int per = (nblocks + nch - 1) / nch;
+    for (int i = threadIdx.x; i < nch * E; i += 256) {
         const int c = i / E, e = i - c * E;
         const int b0 = c * per, b1 = min(nblocks, b0 + per);
         float m = 0.f, n = 0.f;
+#pragma unroll 4
         for (int b = b0; b < b1; ++b) { m += part_me[(size_t)b * E + e]; n += part_cnt[(size_t)b * E + e]; }
         s_m[i] = m;
         s_c[i] = n;
@@ -104,7 +189,7 @@ __global__ __launch_bounds__(256) void router_loss_kernel(float* __restrict__ l_
     float local = 0.f;
     for (int e = threadIdx.x; e < E; e += 256) {
         float m = 0.f, c = 0.f;
-        for (int j = 0; j < 8; ++j) { m += s_m[j * E + e]; c += s_c[j * E + e]; }
+        for (int j = 0; j < nch; ++j) { m += s_m[j * E + e]; c += s_c[j * E + e]; }
         const float cev = c * ((float)E / (float)num_tokens);
         me[e] = m;
         ce[e] = cev;
@@ -173,10 +258,15 @@ extern "C" int hexa_router_forward(float* scores, int32_t* idx, float* me, float
     const int nb = div_up(T, ROUTER_TB);
     float* part_me = ws;
     float* part_cnt = ws + (size_t)nb * E;
-    hipLaunchKernelGGL(router_fwd_kernel, dim3(nb), dim3(ROUTER_TB), sizeof(float) * 2 * E, st, scores, idx, part_me,
-                       part_cnt, logits, noise, noise_scale, T, E, k);
+    if (E <= ROUTER_LDS_E)
+        hipLaunchKernelGGL(router_fwd_kernel<true>, dim3(nb), dim3(ROUTER_TB), sizeof(float) * (2 * E + E * ROUTER_P), st,
+                           scores, idx, part_me, part_cnt, logits, noise, noise_scale, T, E, k);
+    else
+        hipLaunchKernelGGL(router_fwd_kernel<false>, dim3(nb), dim3(ROUTER_TB), sizeof(float) * 2 * E, st, scores, idx,
+                           part_me, part_cnt, logits, noise, noise_scale, T, E, k);
     HEXA_CHECK_LAUNCH("router_fwd");
-    hipLaunchKernelGGL(router_loss_kernel, dim3(1), dim3(256), sizeof(float) * 16 * E, st, l_aux, me, ce, part_me,
+    const int nch = E <= 256 ? 32 : (8192 / E > 0 ? 8192 / E : 1);
+    hipLaunchKernelGGL(router_loss_kernel, dim3(1), dim3(256), sizeof(float) * 2 * nch * E, st, l_aux, me, ce, part_me,
                        part_cnt, nb, T, E);
     HEXA_CHECK_LAUNCH("router_loss");
     return HEXA_OK;

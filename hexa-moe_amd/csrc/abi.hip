@@ -97,7 +97,7 @@ extern "C" int hexa_estmm(void* dw, const void* dy, const void* x, const int32_t
 }
 
 extern "C" int hexa_ess(void* db, const void* dy, const int32_t* route, int dy_per_slot, int accumulate, int T, int k,
-                        int out_dim, int E, int dt, int db_dt, void* stream) {
+                        int out_dim, int E, int dt, int db_dt, float* ws, int64_t ws_floats, void* stream) {
     if (int rc = check_sizes("hexa_ess", T, k, E, out_dim, out_dim)) return rc;
     if (!db || !route || !dy) HEXA_FAIL(HEXA_ERR_ARG, "hexa_ess: null pointer");
     if (!is_dt(dt) || !is_dt(db_dt)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_ess: unknown element type");
@@ -107,6 +107,7 @@ extern "C" int hexa_ess(void* db, const void* dy, const int32_t* route, int dy_p
     a.r = route_view(route, T, k, E);
     a.out_dim = out_dim; a.dy_per_slot = dy_per_slot ? 1 : 0; a.accumulate = accumulate ? 1 : 0;
     a.dy_dt = dt; a.db_dt = db_dt;
+    a.ws = ws; a.ws_floats = ws ? ws_floats : 0;
     return launch_ess(a, st);
 }
 
@@ -124,7 +125,7 @@ extern "C" int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y,
     rc = hexa_estmm(j_w, j_y, x, route, m2s ? 1 : 0, m2s ? 0 : 1, accumulate, T, k, out_dim, in_dim, E, act_dt, jw_dt,
                     stream);
     if (rc) return rc;
-    if (j_b) rc = hexa_ess(j_b, j_y, route, m2s ? 1 : 0, accumulate, T, k, out_dim, E, act_dt, jb_dt, stream);
+    if (j_b) rc = hexa_ess(j_b, j_y, route, m2s ? 1 : 0, accumulate, T, k, out_dim, E, act_dt, jb_dt, nullptr, 0, stream);
     return rc;
 }
 

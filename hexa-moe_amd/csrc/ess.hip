@@ -9,6 +9,8 @@
 // output, bit-reproducible.
 //
 // Replaces the ESS task of fused_grad_bias_kernel_vectorized_* (kernels/fused_ops_full.cu:372-431).
+#include <algorithm>
+
 #include "hexa_internal.h"
 
 namespace hexa {
@@ -23,6 +25,7 @@ struct EssK {
     const void* dy; void* db;
     const int32_t* token_ids; const int32_t* offsets;
     int T, k, E, N, dy_slot_rows, accumulate, db_dt;
+    float* ws; int splits;   // splits > 1: workgroup z sums the z-th part of every segment into ws[z][E][N]
 };
 
 template <typename T>
@@ -44,9 +47,14 @@ __global__ __launch_bounds__(256) void ess_kernel(EssK p) {
 
     bool any = false;
     for (int s = 0; s < p.k; ++s) {
-        const int beg = p.offsets[(size_t)s * (p.E + 1) + e];
-        const int end = p.offsets[(size_t)s * (p.E + 1) + e + 1];
+        int beg = p.offsets[(size_t)s * (p.E + 1) + e];
+        int end = p.offsets[(size_t)s * (p.E + 1) + e + 1];
         any = any || end > beg;
+        if (p.splits > 1) {
+            const int part = (end - beg + p.splits - 1) / p.splits;
+            beg = min(end, beg + (int)blockIdx.z * part);
+            end = min(end, beg + part);
+        }
         const int32_t* tok = p.token_ids + (size_t)s * p.T;
         const T* base = dy + (size_t)p.dy_slot_rows * s * p.N + col;
         // this lane's rows: beg + wave*8 + rg + 32*u + 256*step; the token ids of the next step are
@@ -84,11 +92,23 @@ __global__ __launch_bounds__(256) void ess_kernel(EssK p) {
     __syncthreads();
     if (tid < STRIP) {
         const int c = blockIdx.x * STRIP + tid;
-        if (c < p.N && (any || !p.accumulate)) {
-            const float v = red[0][tid] + red[1][tid] + red[2][tid] + red[3][tid];
+        const float v = red[0][tid] + red[1][tid] + red[2][tid] + red[3][tid];
+        if (p.splits > 1) {
+            if (c < p.N) p.ws[((size_t)blockIdx.z * p.E + e) * p.N + c] = v;
+        } else if (c < p.N && (any || !p.accumulate)) {
             store_out(p.db, (size_t)e * p.N + c, v, p.db_dt, p.accumulate != 0);
         }
     }
+}
+
+// db (+)= ws[0] + ws[1] + ... in that order
+__global__ __launch_bounds__(256) void ess_fold_kernel(void* __restrict__ db, const float* __restrict__ ws, long n,
+                                                       int splits, int db_dt, int accumulate) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float v = ws[i];
+    for (int z = 1; z < splits; ++z) v += ws[(size_t)z * n + i];
+    store_out(db, (size_t)i, v, db_dt, accumulate != 0);
 }
 
 template <typename T>
@@ -101,9 +121,23 @@ int launch_ess_t(const EssArgs& a, hipStream_t st) {
     p.T = a.r.T; p.k = a.r.k; p.E = a.r.E; p.N = a.out_dim;
     p.dy_slot_rows = a.dy_per_slot ? a.r.T : 0;
     p.accumulate = a.accumulate; p.db_dt = a.db_dt;
-    dim3 grid(div_up(a.out_dim, STRIP), a.r.E);
+    // Long token lists are cut into up to 8 parts that run as separate workgroups (the partial sums go
+    // through the caller's scratch and are folded in a fixed order): the kernel is otherwise as slow as
+    // the walk over the busiest expert's list.
+    const long per_part = (long)a.r.E * a.out_dim;
+    const long avg_rows = a.r.E > 0 ? (long)a.r.T * a.r.k / a.r.E : 0;
+    int splits = 1;
+    if (a.ws && per_part > 0 && avg_rows >= 256) splits = (int)std::min<long>(8, a.ws_floats / per_part);
+    if (splits < 2) splits = 1;
+    p.ws = a.ws; p.splits = splits;
+    dim3 grid(div_up(a.out_dim, STRIP), a.r.E, splits);
     hipLaunchKernelGGL((ess_kernel<T>), grid, dim3(256), 0, st, p);
     HEXA_CHECK_LAUNCH("ess");
+    if (splits > 1) {
+        hipLaunchKernelGGL(ess_fold_kernel, dim3((unsigned)((per_part + 255) / 256)), dim3(256), 0, st, a.db, a.ws, per_part,
+                           splits, a.db_dt, a.accumulate);
+        HEXA_CHECK_LAUNCH("ess_fold");
+    }
     return HEXA_OK;
 }
 

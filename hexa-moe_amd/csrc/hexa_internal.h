@@ -69,6 +69,7 @@ struct EssArgs {
     void* db; const void* dy;
     RouteView r;
     int out_dim, dy_per_slot, accumulate, dy_dt, db_dt;
+    float* ws; int64_t ws_floats;   // optional scratch for partial sums
 };
 
 int launch_esmm16(const EsmmArgs& a, hipStream_t s);

@@ -36,7 +36,7 @@ SIGNATURES = {
     "hexa_route_from_lists": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     "hexa_esmm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "hexa_estmm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
-    "hexa_ess": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "hexa_ess": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
     "hexa_fused_grad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "hexa_gelu_bwd": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),
     "hexa_gate_logits": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
@@ -66,7 +66,7 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.hexa_abi_version() != 3:
+    if lib.hexa_abi_version() != 4:
         raise RuntimeError("hexa_moe: libhexa_moe_hip.so has an unexpected ABI version")
     _lib = lib
     return lib

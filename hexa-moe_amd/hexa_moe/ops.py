@@ -221,9 +221,12 @@ def ess(dy, route, dy_per_slot, out=None, out_dtype=torch.float32, accumulate=Fa
     if out is None:
         assert not accumulate
         out = torch.empty(E, out_dim, dtype=out_dtype, device=dy.device)
+    ws = None
+    if T * k >= 256 * E:   # long token lists: scratch for the partial sums of up to 8 parts per list
+        ws = torch.empty(8 * E * out_dim, dtype=torch.float32, device=dy.device)
     rc = _call(f"ess[{out_dim}{',per_slot' if dy_per_slot else ''}]", _lib.load().hexa_ess, _ptr(out), _ptr(dy),
                _ptr(route.blob), int(bool(dy_per_slot)), int(bool(accumulate)), T, k, out_dim, E, _dt(dy), _dt(out),
-               _stream())
+               _ptr(ws), 0 if ws is None else ws.numel(), _stream())
     _lib.check(rc, "hexa_ess")
     return out
 

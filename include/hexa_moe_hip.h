@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define HEXA_ABI_VERSION 3
+#define HEXA_ABI_VERSION 4
 
 /* element types */
 #define HEXA_F32 0
@@ -136,9 +136,12 @@ int hexa_estmm(void* dw, const void* dy, const void* x, const int32_t* route, in
                int dw_dt, void* stream);
 
 /* ESS: db[e][o] (+)= sum over slots and tokens routed to e of dy[(s),t,o].
+ * ws (optional, ws_floats floats of scratch; 8*num_experts*out_dim is enough): long token lists are then
+ * summed in up to 8 parts by separate workgroups and folded in a fixed order, which keeps the kernel
+ * from being as slow as the busiest expert's list; results stay bit-reproducible.
  * Replaces the ESS task of FUSED_GRAD (kernels/fused_ops_full.cu:372-431). */
 int hexa_ess(void* db, const void* dy, const int32_t* route, int dy_per_slot, int accumulate, int num_tokens,
-             int top_k, int out_dim, int num_experts, int dt, int db_dt, void* stream);
+             int top_k, int out_dim, int num_experts, int dt, int db_dt, float* ws, int64_t ws_floats, void* stream);
 
 /* The reference's fused backward of one expert linear:
  *   j_x[(s),t,:in] (+)= j_y[(s),t,:out] . w[e]      w [E][out][in]

@@ -160,6 +160,31 @@ def test_estmm_16bit_result(dev, dtype):
     assert_close(db, O.ess(dy.float(), token_ids, offsets, True, E), TOL[dtype], "ess 16-bit result")
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("per_slot", [False, True])
+def test_ess_long_lists(dev, dtype, per_slot):
+    """Token lists long enough for the split walk (partial sums through scratch, folded in order)."""
+    from hexa_moe import ops
+    T, d_out, E, k = 6000, 200, 8, 2
+    g = gen(91)
+    routing = make_routing(T, E, k, seed=92, skew="zipf", empty=1)
+    _, offsets, token_ids = O.route_build(routing, E)
+    dy = torch.randn((k, T, d_out) if per_slot else (T, d_out), generator=g).to(dtype)
+    rd = _ref_dtype(dtype)
+    want = O.ess(dy.to(rd), token_ids, offsets, per_slot, E)
+    route = ops.route_build(routing.to(dev), E)
+    got = ops.ess(dy.to(dev), route, per_slot)
+    again = ops.ess(dy.to(dev), route, per_slot)
+    torch.cuda.synchronize()
+    assert_close(got, want, TOL[dtype], "ess")
+    assert torch.equal(got, again)
+    base = torch.randn(E, d_out, generator=g)
+    out = base.clone().to(dev)
+    ops.ess(dy.to(dev), route, per_slot, out=out, accumulate=True)
+    torch.cuda.synchronize()
+    assert_close(out, want + base.to(rd), TOL[dtype], "ess accumulate")
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16, F16])
 def test_gelu_bwd(dev, dtype):
     from hexa_moe import ops

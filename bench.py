@@ -138,6 +138,8 @@ def main():
             "gate_logits": ("hbm", T * D * esz + E * D * 4 + T * E * 4),
             "router_forward": ("hbm", 2 * T * E * 4 + T * K_TOP * 4),
             "router_backward": ("hbm", 2 * T * E * 4),
+            "estmm_plan": ("hbm", K_TOP * (E + 1) * 4 + (4 * E + 1) * 4),
+            "gate_backward": ("hbm", T * D * esz * 2 + T * E * 4 + 2 * E * D * 4),
             "gelu_bwd": ("hbm", 3 * T * K_TOP * H * esz),
             f"ess[{H},per_slot]": ("hbm", T * K_TOP * H * esz + E * H * esz),
             f"ess[{D}]": ("hbm", T * K_TOP * D * esz + E * D * esz),

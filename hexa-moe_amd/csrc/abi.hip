@@ -79,7 +79,7 @@ extern "C" int hexa_esmm(void* out, const void* x, const void* w, const void* bi
 
 extern "C" int hexa_estmm(void* dw, const void* dy, const void* x, const int32_t* route, int dy_per_slot,
                           int x_per_slot, int accumulate, int T, int k, int out_dim, int in_dim, int E, int dt,
-                          int dw_dt, void* stream) {
+                          int dw_dt, const int32_t* plan, int max_slots, float* scratch, void* stream) {
     if (int rc = check_sizes("hexa_estmm", T, k, E, in_dim, out_dim)) return rc;
     if (!dw || !route || !dy || !x) HEXA_FAIL(HEXA_ERR_ARG, "hexa_estmm: null pointer");
     if (!is_dt(dt) || !is_dt(dw_dt)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_estmm: unknown element type");
@@ -92,8 +92,17 @@ extern "C" int hexa_estmm(void* dw, const void* dy, const void* x, const int32_t
     a.m_dim = out_dim; a.n_dim = in_dim;
     a.p_per_slot = dy_per_slot ? 1 : 0; a.q_per_slot = x_per_slot ? 1 : 0;
     a.accumulate = accumulate ? 1 : 0; a.pq_dt = dt; a.dw_dt = dw_dt;
+    a.plan = (plan && scratch && max_slots >= 2) ? plan : nullptr;
+    a.max_slots = a.plan ? max_slots : 0;
+    a.scratch = a.plan ? scratch : nullptr;
     if (is_16(dt) && dma_path_enabled() && estmm16_dma_supported(a)) return launch_estmm16_dma(a, st);
     return is_16(dt) ? launch_estmm16(a, st) : launch_estmm32(a, st);
+}
+
+extern "C" int hexa_estmm_plan(int32_t* plan, const int32_t* route, int T, int k, int E, int max_slots, void* stream) {
+    if (int rc = check_sizes("hexa_estmm_plan", T, k, E, 8, 8)) return rc;
+    if (!plan || !route || max_slots < 0) HEXA_FAIL(HEXA_ERR_ARG, "hexa_estmm_plan: bad arguments");
+    return launch_estmm_plan(plan, route_view(route, T, k, E), max_slots, (hipStream_t)stream);
 }
 
 extern "C" int hexa_ess(void* db, const void* dy, const int32_t* route, int dy_per_slot, int accumulate, int T, int k,
@@ -123,7 +132,7 @@ extern "C" int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y,
     if (rc) return rc;
     // ESTMM task: j_w[e][out][in] = sum j_y^T x
     rc = hexa_estmm(j_w, j_y, x, route, m2s ? 1 : 0, m2s ? 0 : 1, accumulate, T, k, out_dim, in_dim, E, act_dt, jw_dt,
-                    stream);
+                    nullptr, 0, nullptr, stream);
     if (rc) return rc;
     if (j_b) rc = hexa_ess(j_b, j_y, route, m2s ? 1 : 0, accumulate, T, k, out_dim, E, act_dt, jb_dt, nullptr, 0, stream);
     return rc;

@@ -25,6 +25,8 @@
 //
 // Constraints of this path (anything else runs on the general kernels of gemm16.hip): operands and
 // weights of one 16-bit type, in_dim a multiple of 32 for ESMM, out/in dims multiples of 8.
+#include <algorithm>
+
 #include "dma_common.h"
 
 namespace hexa {
@@ -286,7 +288,81 @@ struct EstmmK {
     int p_slot_rows, q_slot_rows;
     int accumulate, group;
     long total;
+    const int* plan;     // non-null: units from estmm_plan_kernel (see there); scratch holds the partial results
+    float* scratch;
 };
+
+// ---- plan of a balanced ESTMM launch ------------------------------------------------------------------
+// One workgroup's walk over an expert's token list is serial, so the kernel is as slow as the
+// busiest expert.  With scratch memory, experts with more than `cap` tokens are cut into up to
+// PLAN_MAX_PARTS parts of equal step counts; a part is a unit of work like a whole small expert, its
+// fp32 partial result goes to a scratch slot, and estmm_fixup_kernel adds an expert's slots in order
+// (bit-reproducible).  Units are numbered heaviest expert first.  plan = 4 arrays of E ints in rank
+// order -- expert, parts, first unit, first scratch slot -- followed by the number of units.
+constexpr int PLAN_MAX_PARTS = 4;
+
+__global__ __launch_bounds__(256) void estmm_plan_kernel(int* __restrict__ plan, const int32_t* __restrict__ offsets,
+                                                         int E, int k, int cap, int max_slots) {
+    extern __shared__ int sp[];      // load[E], rank_of[E]  ->  by rank: expert[E], parts[E]
+    int* load = sp;
+    int* expert_of = sp + E;
+    int* parts = sp + 2 * E;
+    for (int e = threadIdx.x; e < E; e += 256) {
+        int t = 0;
+        for (int s = 0; s < k; ++s) t += offsets[(size_t)s * (E + 1) + e + 1] - offsets[(size_t)s * (E + 1) + e];
+        load[e] = t;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += 256) {
+        const int mine = load[e];
+        int r = 0;
+        for (int x = 0; x < E; ++x) {
+            const int o = load[x];
+            r += (o > mine || (o == mine && x < e)) ? 1 : 0;
+        }
+        expert_of[r] = e;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {          // E is small: a serial pass hands out units and scratch slots
+        int unit = 0, slot = 0;
+        for (int r = 0; r < E; ++r) {
+            const int e = expert_of[r];
+            int n = (load[e] + cap - 1) / cap;
+            n = max(1, min(n, PLAN_MAX_PARTS));
+            if (n > 1 && slot + n > max_slots) n = 1;
+            plan[r] = e;
+            plan[E + r] = n;
+            plan[2 * E + r] = unit;
+            plan[3 * E + r] = n > 1 ? slot : -1;
+            unit += n;
+            if (n > 1) slot += n;
+        }
+        plan[4 * E] = unit;
+    }
+}
+
+// dw[e] (+)= slot[0] + slot[1] + ... for the experts that were cut into parts
+__global__ __launch_bounds__(256) void estmm_fixup_kernel(void* __restrict__ dw, const int* __restrict__ plan,
+                                                          const float* __restrict__ scratch, int E, long mn,
+                                                          int dw_dt, int accumulate) {
+    const int r = blockIdx.y;
+    const int n = plan[E + r];
+    if (n <= 1) return;
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= mn) return;
+    const int e = plan[r];
+    const float* src = scratch + (size_t)plan[3 * E + r] * mn + i;
+    float4 v = *reinterpret_cast<const float4*>(src);
+    for (int c = 1; c < n; ++c) {
+        const float4 w = *reinterpret_cast<const float4*>(src + (size_t)c * mn);
+        v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+    }
+    const size_t o = (size_t)e * mn + i;
+    store_out(dw, o, v.x, dw_dt, accumulate != 0);
+    store_out(dw, o + 1, v.y, dw_dt, accumulate != 0);
+    store_out(dw, o + 2, v.z, dw_dt, accumulate != 0);
+    store_out(dw, o + 3, v.w, dw_dt, accumulate != 0);
+}
 
 struct Cursor {   // walks the expert's token list in 32-token steps, slot after slot
     int s, r;
@@ -325,10 +401,20 @@ __global__ __launch_bounds__(C::NT, C::MINW) void estmm16_dma_kernel(EstmmK p) {
     const int M = p.M, N = p.N, T = p.T, nslot = p.k;
 
     // Heaviest experts first: workgroups are dispatched in id order, so giving the long token lists
-    // to the first ones shortens the tail.  The expert of this workgroup is the one whose load has
-    // rank `rank` (ties broken by index).  Up to 256 experts; beyond that the order is by index.
-    int e = rank;
-    if (p.E <= 256) {
+    // to the first ones shortens the tail.  With a plan, `rank` numbers the plan's units (an expert or
+    // one part of a busy expert); without, the expert of this workgroup is the one whose load has rank
+    // `rank` (ties broken by index; up to 256 experts, beyond that the order is by index).
+    int e = rank, part = 0, nparts = 1, slot = -1;
+    if (p.plan) {
+        __shared__ int sUnit[4];
+        if (rank >= p.plan[4 * p.E]) return;
+        for (int r = tid; r < p.E; r += C::NT) {
+            const int u0 = p.plan[2 * p.E + r], n = p.plan[p.E + r];
+            if (rank >= u0 && rank < u0 + n) { sUnit[0] = p.plan[r]; sUnit[1] = rank - u0; sUnit[2] = n; sUnit[3] = p.plan[3 * p.E + r]; }
+        }
+        __syncthreads();
+        e = sUnit[0]; part = sUnit[1]; nparts = sUnit[2]; slot = sUnit[3];
+    } else if (p.E <= 256) {
         __shared__ int sLoad[256];
         if (tid < p.E) {
             int t = 0;
@@ -355,17 +441,21 @@ __global__ __launch_bounds__(C::NT, C::MINW) void estmm16_dma_kernel(EstmmK p) {
         sEnd[tid] = p.offsets[(size_t)tid * (p.E + 1) + e + 1];
     }
     __syncthreads();
-    int nsteps = 0;
-    for (int s = 0; s < nslot; ++s) nsteps += (sEnd[s] - sBeg[s] + BK - 1) / BK;
+    int all_steps = 0;
+    for (int s = 0; s < nslot; ++s) all_steps += (sEnd[s] - sBeg[s] + BK - 1) / BK;
+    // this workgroup's share of the expert's steps (all of them unless the expert was cut into parts)
+    const int step0 = (int)((long)all_steps * part / nparts);
+    const int nsteps = (int)((long)all_steps * (part + 1) / nparts) - step0;
 
-    auto first = [&]() {
-        Cursor c; c.s = 0; c.r = sBeg[0];
-        while (c.s < nslot && c.r >= sEnd[c.s]) { ++c.s; c.r = c.s < nslot ? sBeg[c.s] : 0; }
-        return c;
-    };
     auto advance = [&](Cursor c) {
         c.r += BK;
         while (c.s < nslot && c.r >= sEnd[c.s]) { ++c.s; c.r = c.s < nslot ? sBeg[c.s] : 0; }
+        return c;
+    };
+    auto first = [&]() {
+        Cursor c; c.s = 0; c.r = sBeg[0];
+        while (c.s < nslot && c.r >= sEnd[c.s]) { ++c.s; c.r = c.s < nslot ? sBeg[c.s] : 0; }
+        for (int i = 0; i < step0; ++i) c = advance(c);
         return c;
     };
 
@@ -443,7 +533,7 @@ __global__ __launch_bounds__(C::NT, C::MINW) void estmm16_dma_kernel(EstmmK p) {
             const char* base = smem + (kt % STAGES) * C::STAGE_BYTES;
             mma_stage<TC, C, true, true>(base, base + C::R_BYTES, wr, wf, lane, acc);
         }
-    } else if (p.accumulate) {
+    } else if (p.accumulate && slot < 0) {
         return;
     }
 
@@ -482,6 +572,10 @@ __global__ __launch_bounds__(C::NT, C::MINW) void estmm16_dma_kernel(EstmmK p) {
                 const int m = m0 + h * PRF + ml;
                 if (m >= M || n >= N) continue;
                 float4 v = *reinterpret_cast<const float4*>(sC + ml * CPF + c * 4);
+                if (slot >= 0) {   // one part of a busy expert: fp32 partial result into its scratch slot
+                    *reinterpret_cast<float4*>(p.scratch + ((size_t)(slot + part) * M + m) * N + n) = v;
+                    continue;
+                }
                 const size_t off = ((size_t)e * M + m) * N + n;
                 if (OUT32) {
                     float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(p.dw) + off);
@@ -522,12 +616,28 @@ int launch_estmm_dma_c(const EstmmArgs& a, hipStream_t st) {
     p.q_slot_rows = a.q_per_slot ? a.r.T : 0;
     p.accumulate = a.accumulate;
     p.group = p.ntn * env_int("HEXA_ESTMM_GROUP", 1);
-    p.total = (long)a.r.E * p.mtn * p.ntn;
+    p.plan = nullptr; p.scratch = nullptr;
+    int units = a.r.E;
+    const int E = a.r.E;
+    const long mn = (long)a.m_dim * a.n_dim;
+    if (a.plan && a.scratch && a.max_slots >= 2 && (mn & 3) == 0) {
+        p.plan = a.plan;
+        p.scratch = a.scratch;
+        // every cut adds at most PLAN_MAX_PARTS-1 units and uses at least 2 slots
+        units = E + (int)std::min<long>((long)(a.max_slots / 2) * (PLAN_MAX_PARTS - 1), (long)E * (PLAN_MAX_PARTS - 1));
+    }
+    p.total = (long)units * p.mtn * p.ntn;
     if (p.total == 0) return HEXA_OK;
     const int grid = round_up(p.total, 8 * p.group);
     const bool o32 = a.dw_dt == HEXA_F32;
-    if (a.pq_dt == HEXA_BF16) return o32 ? launch_estmm_dma_t<__bf16, true, C>(p, grid, st) : launch_estmm_dma_t<__bf16, false, C>(p, grid, st);
-    return o32 ? launch_estmm_dma_t<_Float16, true, C>(p, grid, st) : launch_estmm_dma_t<_Float16, false, C>(p, grid, st);
+    int rc;
+    if (a.pq_dt == HEXA_BF16) rc = o32 ? launch_estmm_dma_t<__bf16, true, C>(p, grid, st) : launch_estmm_dma_t<__bf16, false, C>(p, grid, st);
+    else rc = o32 ? launch_estmm_dma_t<_Float16, true, C>(p, grid, st) : launch_estmm_dma_t<_Float16, false, C>(p, grid, st);
+    if (rc || !p.plan) return rc;
+    hipLaunchKernelGGL(estmm_fixup_kernel, dim3((unsigned)((mn / 4 + 255) / 256), E), dim3(256), 0, st, a.dw, p.plan, p.scratch,
+                       E, mn, a.dw_dt, a.accumulate);
+    HEXA_CHECK_LAUNCH("estmm_fixup");
+    return HEXA_OK;
 }
 
 template <typename C>
@@ -586,6 +696,16 @@ int pick_esmm_tile(long rows, int cols, int in_dim) {
 
 }  // namespace
 
+int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, hipStream_t st) {
+    if (r.E > 4096) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "estmm plan: more than 4096 experts");
+    const long avg = (long)r.T * r.k / r.E;
+    const int cap = (int)std::max<long>(256, (3 * avg + 1) / 2);   // parts for experts above 1.5x the mean load
+    hipLaunchKernelGGL(estmm_plan_kernel, dim3(1), dim3(256), 3 * r.E * sizeof(int), st, plan, r.offsets, r.E, r.k, cap,
+                       max_slots);
+    HEXA_CHECK_LAUNCH("estmm_plan");
+    return HEXA_OK;
+}
+
 bool esmm16_dma_supported(const EsmmArgs& a) {
     return a.w_dt == a.x_dt && (a.in_dim % 32) == 0 && (a.out_dim % 8) == 0 &&
            (a.out_dt == a.x_dt || a.out_dt == HEXA_F32);
@@ -608,7 +728,9 @@ int launch_estmm16_dma(const EstmmArgs& a, hipStream_t st) {
         case 6: return launch_estmm_dma_c<CfgX16>(a, st);
         case 8: return launch_estmm_dma_c<CfgS2>(a, st);
         case 9: return launch_estmm_dma_c<CfgS3>(a, st);
-        default: return launch_estmm_dma_c<CfgS>(a, st);
+        case 1: return launch_estmm_dma_c<CfgS>(a, st);
+        // balanced units (a plan) keep 4 workgroups per CU busy; without a plan, more LDS per workgroup wins
+        default: return a.plan ? launch_estmm_dma_c<CfgS2>(a, st) : launch_estmm_dma_c<CfgS>(a, st);
     }
 }
 

@@ -64,6 +64,7 @@ struct EstmmArgs {
     int p_per_slot, q_per_slot;
     int accumulate;
     int pq_dt, dw_dt;
+    const int32_t* plan; int max_slots; float* scratch;   // optional: the busiest experts cut into parts
 };
 struct EssArgs {
     void* db; const void* dy;
@@ -76,6 +77,7 @@ int launch_esmm16(const EsmmArgs& a, hipStream_t s);
 int launch_esmm32(const EsmmArgs& a, hipStream_t s);
 bool esmm16_dma_supported(const EsmmArgs& a);
 bool esmm16_persist_supported(const EsmmArgs& a);
+int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, hipStream_t st);
 int launch_esmm16_persist(const EsmmArgs& a, int tile, hipStream_t st);
 int launch_esmm16_dma(const EsmmArgs& a, hipStream_t s);
 bool dma_path_enabled();

@@ -71,6 +71,19 @@ class Route:
     def __init__(self, blob, T, k, E):
         self.blob, self.T, self.k, self.E = blob, int(T), int(k), int(E)
         self.layout = _lib.route_layout(T, k, E)
+        self._plans = {}
+
+    def estmm_plan(self, max_slots):
+        """Work plan of estmm for this routing (int32 [4E+1]); made on first use, then shared by every
+        estmm call on the routing."""
+        plan = self._plans.get(max_slots)
+        if plan is None:
+            plan = torch.empty(4 * self.E + 1, dtype=torch.int32, device=self.blob.device)
+            rc = _call("estmm_plan", _lib.load().hexa_estmm_plan, _ptr(plan), _ptr(self.blob), self.T, self.k, self.E,
+                       int(max_slots), _stream())
+            _lib.check(rc, "hexa_estmm_plan")
+            self._plans[max_slots] = plan
+        return plan
 
     def _part(self, start, n):
         return self.blob[start:start + n]
@@ -204,9 +217,18 @@ def estmm(dy, x, route, dy_per_slot, x_per_slot, out=None, out_dtype=torch.float
     if out is None:
         assert not accumulate
         out = torch.empty(E, out_dim, in_dim, dtype=out_dtype, device=x.device)
+    plan = scratch = None
+    slots = 0
+    if x.dtype != torch.float32 and T * k >= 128 * E:
+        # the busiest experts are cut into parts: a plan (made once per routing) and scratch for up to 2E fp32
+        # partial results, at most 256 MiB
+        slots = min(2 * E, (256 << 20) // (out_dim * in_dim * 4))
+        if slots >= 2 and (out_dim * in_dim) % 4 == 0:
+            plan = route.estmm_plan(slots)
+            scratch = torch.empty(slots * out_dim * in_dim, dtype=torch.float32, device=x.device)
     rc = _call(f"estmm[{out_dim}x{in_dim}]", _lib.load().hexa_estmm, _ptr(out), _ptr(dy), _ptr(x), _ptr(route.blob),
                int(bool(dy_per_slot)), int(bool(x_per_slot)), int(bool(accumulate)), T, k, out_dim, in_dim, E,
-               _dt(x), _dt(out), _stream())
+               _dt(x), _dt(out), _ptr(plan), slots if plan is not None else 0, _ptr(scratch), _stream())
     _lib.check(rc, "hexa_estmm")
     return out
 

@@ -130,10 +130,23 @@ int hexa_esmm(void* out, const void* x, const void* w, const void* bias, const i
  * dy_per_slot / x_per_slot say whether the operand is [k,T,*] (1) or [T,*] shared by the slots (0).
  * dt is the element type of dy and x (F32, F16 or BF16); dw_dt is F32 or dt.  Experts without tokens
  * get exact zeros (or are left untouched when accumulating).
+ * plan / max_slots / scratch (optional; used by the 16-bit kernels): with a plan from hexa_estmm_plan for
+ * the same routing and max_slots, experts with more than 1.5x the mean number of tokens are cut into up
+ * to 4 parts that run as separate workgroups; the fp32 partial results go through `scratch`
+ * (max_slots * out_dim * in_dim floats) and are added in a fixed order, so results stay bit-reproducible.
+ * Without it one workgroup walks an expert's whole token list and the kernel is as slow as the busiest
+ * expert.
  * Replaces the ESTMM task of FUSED_GRAD (kernels/fused_ops_full.cu:248-371). */
 int hexa_estmm(void* dw, const void* dy, const void* x, const int32_t* route, int dy_per_slot, int x_per_slot,
                int accumulate, int num_tokens, int top_k, int out_dim, int in_dim, int num_experts, int dt,
-               int dw_dt, void* stream);
+               int dw_dt, const int32_t* plan, int max_slots, float* scratch, void* stream);
+
+/* Work plan of hexa_estmm for one routing: 4*num_experts+1 ints (experts by decreasing load, their parts,
+ * first work unit and first scratch slot, number of units).  Depends on the routing and max_slots only, so one
+ * plan serves every hexa_estmm call of a layer's backward.  No counterpart in the reference, whose ESTMM
+ * task walks each expert's list in one thread block (kernels/fused_ops_full.cu:248-371). */
+int hexa_estmm_plan(int32_t* plan, const int32_t* route, int num_tokens, int top_k, int num_experts, int max_slots,
+                    void* stream);
 
 /* ESS: db[e][o] (+)= sum over slots and tokens routed to e of dy[(s),t,o].
  * ws (optional, ws_floats floats of scratch; 8*num_experts*out_dim is enough): long token lists are then

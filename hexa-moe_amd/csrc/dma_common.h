@@ -226,12 +226,16 @@ template <typename TC> __device__ __forceinline__ uint2 pack4(float a, float b, 
     return o;
 }
 
-// GELU (erf form) with erf from Abramowitz & Stegun 7.1.26 (|error| < 1.5e-7): one exp, one
-// reciprocal and a degree-5 polynomial instead of the library erff.  Used where the result is rounded
-// to 16 bits (or compared at 2e-2); the fp32 kernels keep erff.
+// GELU (erf form) with erf from Abramowitz & Stegun 7.1.26 (|error| < 1.5e-7): one exp2, one hardware
+// reciprocal and a degree-5 polynomial instead of the library erff (whose division alone is a dozen
+// instructions).  The epilogue's arithmetic is not free here: a wavefront's VALU instruction occupies
+// its SIMD for 4 cycles (16 for the transcendental ones), and at a contraction length of a few hundred
+// a tile's epilogue costs about as many SIMD cycles as its MFMAs.  Used where the result is rounded to
+// 16 bits (or compared at 2e-2); the fp32 kernels keep erff.  (An 8-term odd polynomial for erf,
+// FMAs only, was measured too: 5 % faster on the fused fc1 launch at 1.5e-4 error -- not taken.)
 __device__ __forceinline__ float gelu_fast(float x) {
     const float z = fabsf(x) * 0.70710678118654752440f;
-    const float t = __frcp_rn(1.0f + 0.3275911f * z);
+    const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
     const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
     const float erf_abs = 1.0f - poly * __expf(-z * z);
     const float erf_x = copysignf(erf_abs, x);
@@ -241,7 +245,7 @@ __device__ __forceinline__ float gelu_fast(float x) {
 // gelu'(x) = Phi(x) + x*phi(x) with the same erf approximation (shares its exponential)
 __device__ __forceinline__ float gelu_grad_fast(float x) {
     const float z = fabsf(x) * 0.70710678118654752440f;
-    const float t = __frcp_rn(1.0f + 0.3275911f * z);
+    const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
     const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
     const float ex = __expf(-z * z);
     const float erf_x = copysignf(1.0f - poly * ex, x);
@@ -257,6 +261,7 @@ struct EsmmK {
     int T, K, N, mt_ub, ntn, slot_begin, nslots;
     int x_slot_rows, out_slot_rows;
     int accumulate, bias_dt, out_dt, act, group;
+    int stream_out;   // results are stored with the streaming (non-temporal) hint
     long total;
     void* ws;   // slots > 0 write here ([slot-1][T][N]) when set: the slots are summed afterwards
 };

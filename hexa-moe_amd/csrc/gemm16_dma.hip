@@ -32,6 +32,16 @@
 namespace hexa {
 namespace {
 
+// 16-byte store; `streaming` marks the line as not worth keeping in the caches (results that are much
+// larger than the L2 would otherwise push the weights and token rows out of it)
+__device__ __forceinline__ void store16(uint4* dst, uint4 v, bool streaming) {
+    typedef __attribute__((ext_vector_type(4))) unsigned u4;
+    u4 w;
+    w.x = v.x; w.y = v.y; w.z = v.z; w.w = v.w;
+    if (streaming) __builtin_nontemporal_store(w, reinterpret_cast<u4*>(dst));
+    else *reinterpret_cast<u4*>(dst) = w;
+}
+
 template <typename TC, bool W_IN_OUT, bool OUT32, typename C>
 __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
     constexpr int BM = C::BM, BN = C::BN, STAGES = C::STAGES, NW = C::NW, BK = C::BKC;
@@ -236,7 +246,7 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
                         }
                         val = make_uint4(vw[0], vw[1], vw[2], vw[3]);
                     }
-                    *dst = val;
+                    store16(dst, val, p.stream_out == 1);
                     if (gelu) {
                         // applied to the value as stored (rounded), like act(y1) on the tensor
                         unsigned vw[4] = {val.x, val.y, val.z, val.w};
@@ -244,8 +254,8 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
                         for (int q = 0; q < 4; ++q)
                             vw[q] = bits16<TC>(gelu_fast(from_bits16<TC>(vw[q] & 0xffff))) |
                                     ((unsigned)bits16<TC>(gelu_fast(from_bits16<TC>(vw[q] >> 16))) << 16);
-                        *reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(p.out_act) + off) =
-                            make_uint4(vw[0], vw[1], vw[2], vw[3]);
+                        store16(reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(p.out_act) + off),
+                                make_uint4(vw[0], vw[1], vw[2], vw[3]), p.stream_out == 1);
                     }
                 }
             }
@@ -653,6 +663,7 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
     p.x_slot_rows = a.x_per_slot ? a.r.T : 0;
     p.out_slot_rows = a.out_per_slot ? a.r.T : 0;
     p.bias_dt = a.bias_dt; p.out_dt = a.out_dt; p.act = a.act;
+    p.stream_out = env_int("HEXA_ESMM_STREAM", 0);
     p.group = p.ntn * env_int("HEXA_ESMM_GROUP", large ? 2 : 4);
     // Summing the slots into one result: with scratch, every slot runs in ONE launch (slot 0 into
     // `out`, the others into the scratch) and a reduction adds them in slot order; without it, one

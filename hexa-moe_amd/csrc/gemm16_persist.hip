@@ -677,7 +677,7 @@ int launch_c(const EsmmArgs& a, bool large, hipStream_t st) {
     p.x_slot_rows = a.x_per_slot ? a.r.T : 0;
     p.out_slot_rows = a.out_per_slot ? a.r.T : 0;
     p.bias_dt = a.bias_dt; p.out_dt = a.out_dt; p.act = a.act;
-    p.group = 0; p.total = 0;
+    p.group = 0; p.total = 0; p.stream_out = 0;
     // Summing the slots into one result: with scratch, every slot runs in ONE launch (slot 0 into
     // `out`, the others into the scratch) and a reduction adds them in slot order; without it, one
     // launch per slot, each adding into `out`.

@@ -17,11 +17,26 @@ void set_error(const char* fmt, ...) {
     va_end(ap);
 }
 
-// HEXA_MOE_GENERAL_KERNELS=1 forces the general kernels (testing aid; read once).
-bool dma_path_enabled() {
-    static const bool on = [] { const char* v = getenv("HEXA_MOE_GENERAL_KERNELS"); return !(v && v[0] == '1'); }();
-    return on;
+namespace {
+struct OptEntry { const char* name; const char* env; int value; bool loaded; };
+OptEntry g_opts[OPT_COUNT] = {
+    {"tile", "HEXA_MOE_TILE", 0, false},          {"persist", "HEXA_MOE_PERSIST", 0, false},
+    {"general_kernels", "HEXA_MOE_GENERAL_KERNELS", 0, false}, {"esmm_map", "HEXA_ESMM_MAP", 0, false},
+    {"esmm_group", "HEXA_ESMM_GROUP", 0, false},  {"estmm_group", "HEXA_ESTMM_GROUP", 0, false},
+    {"esmm_stream", "HEXA_ESMM_STREAM", 0, false},
+};
+}  // namespace
+
+int option(int id) {
+    OptEntry& o = g_opts[id];
+    if (!o.loaded) {
+        const char* v = getenv(o.env);
+        o.value = v ? atoi(v) : 0;
+        o.loaded = true;
+    }
+    return o.value;
 }
+bool dma_path_enabled() { return option(OPT_GENERAL) != 1; }
 
 static bool is_dt(int dt) { return dt == HEXA_F32 || dt == HEXA_F16 || dt == HEXA_BF16; }
 static bool is_16(int dt) { return dt == HEXA_F16 || dt == HEXA_BF16; }
@@ -35,6 +50,18 @@ static int check_sizes(const char* who, int T, int k, int E, int a, int b) {
 }  // namespace hexa
 
 using namespace hexa;
+
+extern "C" int hexa_set_option(const char* name, int value) {
+    if (!name) HEXA_FAIL(HEXA_ERR_ARG, "hexa_set_option: null name");
+    for (int i = 0; i < OPT_COUNT; ++i)
+        if (!strcmp(name, g_opts[i].name)) {
+            g_opts[i].value = value;
+            g_opts[i].loaded = true;
+            return HEXA_OK;
+        }
+    HEXA_FAIL(HEXA_ERR_ARG, "hexa_set_option: unknown option '%s'", name);
+}
+
 
 extern "C" const char* hexa_last_error(void) { return g_err; }
 extern "C" int hexa_abi_version(void) { return HEXA_ABI_VERSION; }

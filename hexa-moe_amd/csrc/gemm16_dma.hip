@@ -263,12 +263,6 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
     }
 }
 
-// integer tuning knob from the environment (read on every call: testing aid only)
-static int env_int(const char* name, int dflt) {
-    const char* s = getenv(name);
-    return s ? atoi(s) : dflt;
-}
-
 template <typename TC, bool IO, bool OUT32, typename C>
 int launch_esmm_dma_t(EsmmK& p, int grid, hipStream_t st) {
     auto kernel = esmm16_dma_kernel<TC, IO, OUT32, C>;
@@ -625,7 +619,7 @@ int launch_estmm_dma_c(const EstmmArgs& a, hipStream_t st) {
     p.p_slot_rows = a.p_per_slot ? a.r.T : 0;
     p.q_slot_rows = a.q_per_slot ? a.r.T : 0;
     p.accumulate = a.accumulate;
-    p.group = p.ntn * env_int("HEXA_ESTMM_GROUP", 1);
+    p.group = p.ntn * std::max(1, option(OPT_ESTMM_GROUP));
     p.plan = nullptr; p.scratch = nullptr;
     int units = a.r.E;
     const int E = a.r.E;
@@ -663,8 +657,8 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
     p.x_slot_rows = a.x_per_slot ? a.r.T : 0;
     p.out_slot_rows = a.out_per_slot ? a.r.T : 0;
     p.bias_dt = a.bias_dt; p.out_dt = a.out_dt; p.act = a.act;
-    p.stream_out = env_int("HEXA_ESMM_STREAM", 0);
-    p.group = p.ntn * env_int("HEXA_ESMM_GROUP", large ? 2 : 4);
+    p.stream_out = option(OPT_ESMM_STREAM) == 1;
+    p.group = p.ntn * (option(OPT_ESMM_GROUP) > 0 ? option(OPT_ESMM_GROUP) : (large ? 2 : 4));
     // Summing the slots into one result: with scratch, every slot runs in ONE launch (slot 0 into
     // `out`, the others into the scratch) and a reduction adds them in slot order; without it, one
     // launch per slot, each adding into `out`.
@@ -677,7 +671,7 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
         p.accumulate = (a.accumulate || l > 0) ? 1 : 0;
         p.total = (long)p.nslots * p.mt_ub * p.ntn;
         if (p.total == 0) continue;
-        const bool contiguous = p.nslots <= 8 && env_int("HEXA_ESMM_MAP", 0) == 1;
+        const bool contiguous = p.nslots <= 8 && option(OPT_ESMM_MAP) == 1;
         const int grid = round_up(p.total, contiguous ? 8 : 8 * p.group);
         if (contiguous) p.group = 0;
         const bool io = a.w_layout == HEXA_W_IN_OUT;
@@ -693,10 +687,7 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
 // HEXA_MOE_TILE (testing aid, read once): 0 automatic; 1 128x128; 2 256x128 (8 wavefronts); 3 256x128
 // (4 wavefronts); 4..6 256x256 (4 / 8 / 16 wavefronts); 7 128x384; 8, 9 128x128 with 4 / 3 workgroups
 // per CU; 10, 11 128x128 / 256x128 with 64 contraction indices per stage (ESMM only)
-int forced_tile() {
-    static const int v = [] { const char* s = getenv("HEXA_MOE_TILE"); return s ? atoi(s) : 0; }();
-    return v;
-}
+int forced_tile() { return option(OPT_TILE); }
 
 int pick_esmm_tile(long rows, int cols, int in_dim) {
     const int f = forced_tile();
@@ -747,10 +738,7 @@ int launch_estmm16_dma(const EstmmArgs& a, hipStream_t st) {
 
 // HEXA_MOE_PERSIST=1 selects the persistent-workgroup ESMM kernels (read once).  They are parity-
 // tested but not the default: on the shapes measured so far the one-tile-per-workgroup kernels win.
-static bool persist_enabled() {
-    static const bool v = [] { const char* s = getenv("HEXA_MOE_PERSIST"); return s && atoi(s) != 0; }();
-    return v;
-}
+static bool persist_enabled() { return option(OPT_PERSIST) == 1; }
 
 int launch_esmm16_dma(const EsmmArgs& a, hipStream_t st) {
     if (persist_enabled() && esmm16_persist_supported(a)) return launch_esmm16_persist(a, forced_tile(), st);

@@ -75,6 +75,20 @@ struct EssArgs {
 
 int launch_esmm16(const EsmmArgs& a, hipStream_t s);
 int launch_esmm32(const EsmmArgs& a, hipStream_t s);
+// Tuning / testing knobs: 0 = automatic.  Each one starts from an environment variable (read once) and
+// can be changed at run time with hexa_set_option.
+enum Opt {
+    OPT_TILE,           // HEXA_MOE_TILE: tile configuration of the 16-bit fast path (see gemm16_dma.hip)
+    OPT_PERSIST,        // HEXA_MOE_PERSIST: 1 = persistent-workgroup ESMM kernels
+    OPT_GENERAL,        // HEXA_MOE_GENERAL_KERNELS: 1 = general 16-bit kernels instead of the fast path
+    OPT_ESMM_MAP,       // HEXA_ESMM_MAP: 1 = every XCD walks one contiguous eighth of the tiles
+    OPT_ESMM_GROUP,     // HEXA_ESMM_GROUP: row tiles per XCD run
+    OPT_ESTMM_GROUP,    // HEXA_ESTMM_GROUP: row tiles per XCD run
+    OPT_ESMM_STREAM,    // HEXA_ESMM_STREAM: 1 = results stored with the streaming hint
+    OPT_COUNT
+};
+int option(int id);
+
 bool esmm16_dma_supported(const EsmmArgs& a);
 bool esmm16_persist_supported(const EsmmArgs& a);
 int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, hipStream_t st);

@@ -48,6 +48,7 @@ SIGNATURES = {
     "hexa_router_backward": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "hexa_last_error": (ctypes.c_char_p, []),
     "hexa_abi_version": (_i, []),
+    "hexa_set_option": (_i, [ctypes.c_char_p, _i]),
 }
 
 _lib = None

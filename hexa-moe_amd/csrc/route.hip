@@ -134,14 +134,54 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ u
     int* tmp = tbase + (E + 1);
     const int s = blockIdx.x;
     int32_t* H = unit_hist + (size_t)s * units * E;
-    for (int e = threadIdx.x; e < E; e += 256) {
-        int run = 0;
-        for (int u = 0; u < units; ++u) {
-            int c = H[(size_t)u * E + e];
-            H[(size_t)u * E + e] = run;
-            run += c;
+    // Exclusive prefix over the units, per expert.  Up to 256 experts: 256/E threads share an expert,
+    // each takes a contiguous range of units (sum, then rewrite), and loads go 8 at a time so that the
+    // memory latency is paid once per batch, not once per unit.
+    __shared__ int32_t part[256];
+    const int G = E <= 256 ? 256 / E : 1;
+    for (int e0 = 0; e0 < E; e0 += 256) {
+        const int tid = threadIdx.x;
+        const int e = G > 1 ? tid % E : e0 + tid;
+        const int j = G > 1 ? tid / E : 0;
+        const bool active = e < E && j < G;
+        const int per = (units + G - 1) / G;
+        const int u_begin = min(units, j * per), u_end = min(units, u_begin + per);
+        int sum = 0;
+        if (active) {
+            for (int u0 = u_begin; u0 < u_end; u0 += 8) {
+                int c[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) c[i] = u0 + i < u_end ? H[(size_t)(u0 + i) * E + e] : 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) sum += c[i];
+            }
         }
-        tot[e] = run;
+        if (G > 1) {
+            part[tid] = active ? sum : 0;
+            __syncthreads();
+        }
+        int run = 0;
+        if (active) {
+            for (int q = 0; q < j; ++q) run += part[q * E + e];
+            if (G > 1 && j == 0) {
+                int t = 0;
+                for (int q = 0; q < G; ++q) t += part[q * E + e];
+                tot[e] = t;
+            } else if (G == 1) {
+                tot[e] = sum;
+            }
+            for (int u0 = u_begin; u0 < u_end; u0 += 8) {
+                int c[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) c[i] = u0 + i < u_end ? H[(size_t)(u0 + i) * E + e] : 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (u0 + i < u_end) H[(size_t)(u0 + i) * E + e] = run;
+                    run += c[i];
+                }
+            }
+        }
+        if (G > 1) break;
     }
     __syncthreads();
     if (prefix_only) return;

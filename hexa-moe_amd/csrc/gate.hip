@@ -30,15 +30,20 @@ __device__ __forceinline__ f32x16 zero16() {
     return z;
 }
 
-// N consecutive elements (N = 4 or 8) as floats; zeros when !ok
+__device__ __attribute__((aligned(32))) unsigned int g_gate_zeros[8];   // stays zero: what masked lanes load
+
+// N consecutive elements (N = 4 or 8) as floats; zeros when !ok.  Masked lanes load from a block of
+// zeros instead of branching around the load, so that a run of loads is issued back to back and
+// their latencies overlap.
 template <typename T, int N> struct LoadN {   // 16-bit types
     static __device__ __forceinline__ void run(const T* p, bool ok, float (&o)[N]) {
+        const T* src = ok ? p : reinterpret_cast<const T*>(g_gate_zeros);
         union { unsigned u[N / 2]; T h[N]; } v;
         if (N == 8) {
-            const uint4 w = ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0u, 0u, 0u, 0u);
+            const uint4 w = *reinterpret_cast<const uint4*>(src);
             v.u[0] = w.x; v.u[1] = w.y; v.u[N / 2 - 2] = w.z; v.u[N / 2 - 1] = w.w;
         } else {
-            const uint2 w = ok ? *reinterpret_cast<const uint2*>(p) : make_uint2(0u, 0u);
+            const uint2 w = *reinterpret_cast<const uint2*>(src);
             v.u[0] = w.x; v.u[1] = w.y;
         }
 #pragma unroll
@@ -47,13 +52,33 @@ template <typename T, int N> struct LoadN {   // 16-bit types
 };
 template <int N> struct LoadN<float, N> {
     static __device__ __forceinline__ void run(const float* p, bool ok, float (&o)[N]) {
+        const float* src = ok ? p : reinterpret_cast<const float*>(g_gate_zeros);
 #pragma unroll
         for (int q = 0; q < N; q += 4) {
-            const float4 v = ok ? *reinterpret_cast<const float4*>(p + q) : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float4 v = *reinterpret_cast<const float4*>(src + q);
             o[q] = v.x; o[q + 1] = v.y; o[q + 2] = v.z; o[q + 3] = v.w;
         }
     }
 };
+// All of v[] has arrived before anything behind this point runs: keeps the scheduler from sinking each
+// load next to its first use (which would pay one memory latency per load instead of one per batch).
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+template <int N> __device__ __forceinline__ void arrive(float (&v)[N][4]) {
+    static_assert(N == 8 || N == 16, "batches of 8 or 16");
+    f32x4 w[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) { w[i].x = v[i][0]; w[i].y = v[i][1]; w[i].z = v[i][2]; w[i].w = v[i][3]; }
+    if constexpr (N == 16)
+        asm volatile("" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]), "+v"(w[4]), "+v"(w[5]), "+v"(w[6]), "+v"(w[7]),
+                          "+v"(w[8]), "+v"(w[9]), "+v"(w[10]), "+v"(w[11]), "+v"(w[12]), "+v"(w[13]), "+v"(w[14]), "+v"(w[15]));
+    else
+        asm volatile("" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]), "+v"(w[4]), "+v"(w[5]), "+v"(w[6]), "+v"(w[7]));
+#pragma unroll
+    for (int i = 0; i < N; ++i) { v[i][0] = w[i].x; v[i][1] = w[i].y; v[i][2] = w[i].z; v[i][3] = w[i].w; }
+}
+__device__ __forceinline__ float load1(const float* p, bool ok) {
+    return *(ok ? p : reinterpret_cast<const float*>(g_gate_zeros));
+}
 template <typename T> __device__ __forceinline__ void store4(T* p, float a, float b, float c, float d);
 template <> __device__ __forceinline__ void store4<float>(float* p, float a, float b, float c, float d) {
     *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
@@ -123,29 +148,32 @@ __global__ __launch_bounds__(256) void gate_dx_kernel(T* __restrict__ dx, const 
         f32x16 acc[4] = {zero16(), zero16(), zero16(), zero16()};
         for (int e0 = 0; e0 < E; e0 += 32) {
             // this lane's contraction indices: experts e0 + 16h + 0..15
-            float a[16];
+            float a[16], b[16][4];
             if ((E & 3) == 0) {   // rows are 16-byte aligned: four float4 loads
 #pragma unroll
                 for (int i = 0; i < 16; i += 4) {
                     const int e = e0 + 16 * h + i;
-                    const float4 v = (tok_ok && e < E) ? *reinterpret_cast<const float4*>(drow + e) : make_float4(0.f, 0.f, 0.f, 0.f);
-                    a[i] = v.x; a[i + 1] = v.y; a[i + 2] = v.z; a[i + 3] = v.w;
+                    float v[4];
+                    LoadN<float, 4>::run(drow + e, tok_ok && e < E, v);
+                    a[i] = v[0]; a[i + 1] = v[1]; a[i + 2] = v[2]; a[i + 3] = v[3];
                 }
             } else {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int e = e0 + 16 * h + i;
-                    a[i] = (tok_ok && e < E) ? drow[e] : 0.f;
+                    a[i] = load1(drow + e, tok_ok && e < E);
                 }
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int e = e0 + 16 * h + i;
-                float b[4];
-                LoadN<float, 4>::run(wg + (size_t)e * d + col, col_ok && e < E, b);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[j], 0, 0, 0);
+                LoadN<float, 4>::run(wg + (size_t)e * d + col, col_ok && e < E, b[i]);
             }
+            arrive(b);
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[i][j], acc[j], 0, 0, 0);
         }
         if (col_ok) {
 #pragma unroll
@@ -172,15 +200,20 @@ __global__ __launch_bounds__(256) void gate_dwg_kernel(float* __restrict__ part,
         const int col = g * 128 + 4 * r;
         const bool col_ok = col < d;
         f32x16 acc[4] = {zero16(), zero16(), zero16(), zero16()};
-#pragma unroll 8
-        for (int i = 0; i < DWG_TB / 2; ++i) {
-            const int t = t0 + 2 * i + h;          // this lane's contraction index: one token
-            const bool ok = t < num_tokens;
-            const float a = (ok && exp_ok) ? dl[(size_t)t * E + e0 + r] : 0.f;
-            float b[4];
-            LoadN<T, 4>::run(x + (size_t)t * d + col, ok && col_ok, b);
+        for (int i0 = 0; i0 < DWG_TB / 2; i0 += 8) {
+            float a[8], b[8][4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b[j], acc[j], 0, 0, 0);
+            for (int u = 0; u < 8; ++u) {
+                const int t = t0 + 2 * (i0 + u) + h;          // this lane's contraction index: one token
+                const bool ok = t < num_tokens;
+                a[u] = load1(dl + (size_t)t * E + e0 + r, ok && exp_ok);
+                LoadN<T, 4>::run(x + (size_t)t * d + col, ok && col_ok, b[u]);
+            }
+            arrive(b);
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u][j], acc[j], 0, 0, 0);
         }
         if (col_ok) {
 #pragma unroll

@@ -307,10 +307,9 @@ constexpr int PLAN_MAX_PARTS = 4;
 
 __global__ __launch_bounds__(256) void estmm_plan_kernel(int* __restrict__ plan, const int32_t* __restrict__ offsets,
                                                          int E, int k, int cap, int max_slots) {
-    extern __shared__ int sp[];      // load[E], rank_of[E]  ->  by rank: expert[E], parts[E]
+    extern __shared__ int sp[];      // load[E], expert_of[E] (the expert at each rank)
     int* load = sp;
     int* expert_of = sp + E;
-    int* parts = sp + 2 * E;
     for (int e = threadIdx.x; e < E; e += 256) {
         int t = 0;
         for (int s = 0; s < k; ++s) t += offsets[(size_t)s * (E + 1) + e + 1] - offsets[(size_t)s * (E + 1) + e];

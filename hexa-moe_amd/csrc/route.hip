@@ -266,6 +266,44 @@ __global__ __launch_bounds__(256) void route_from_lists_kernel(const int32_t* __
                 tile_count_l + s, mt_ub_l);
 }
 
+// Padded lists -> exact lists.  One workgroup per slot walks the slot's stretch of the concatenated
+// lists ([slot_ends[s], slot_ends[s+1]) ) and keeps, in order, every entry whose token id is in range;
+// fillers (-1) drop out.  Positions past the last kept entry get token -1 / expert E, which the
+// operators never visit (they sit beyond offsets[E]).
+__global__ __launch_bounds__(1024) void route_compact_kernel(const int32_t* __restrict__ tok_in,
+                                                             const int32_t* __restrict__ exp_in,
+                                                             const int32_t* __restrict__ slot_ends, int64_t list_len,
+                                                             int T, int E, int32_t* __restrict__ tok_out,
+                                                             int32_t* __restrict__ exp_out) {
+    __shared__ int wave_tot[16];
+    __shared__ int base_sh;
+    const int s = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    int64_t begin = slot_ends[s], end = slot_ends[s + 1];
+    if (begin < 0) begin = 0;
+    if (end > list_len) end = list_len;
+    int32_t* to = tok_out + (size_t)s * T;
+    int32_t* eo = exp_out + (size_t)s * T;
+    if (threadIdx.x == 0) base_sh = 0;
+    __syncthreads();
+    for (int64_t c = begin; c < end; c += 1024) {
+        const int64_t i = c + threadIdx.x;
+        int32_t t = -1, e = 0;
+        if (i < end) { t = tok_in[i]; e = exp_in[i]; }
+        const bool keep = t >= 0 && t < T && e >= 0 && e < E;
+        const unsigned long long m = __ballot(keep);
+        if (lane == 0) wave_tot[wv] = __popcll(m);
+        __syncthreads();
+        int before = base_sh;
+        for (int w = 0; w < wv; ++w) before += wave_tot[w];
+        const int pos = before + __popcll(m & ((1ull << lane) - 1));
+        if (keep && pos < T) { to[pos] = t; eo[pos] = e; }
+        __syncthreads();
+        if (threadIdx.x == 0) { int tot = 0; for (int w = 0; w < 16; ++w) tot += wave_tot[w]; base_sh += tot; }
+        __syncthreads();
+    }
+    for (int p = base_sh + threadIdx.x; p < T; p += 1024) { to[p] = -1; eo[p] = E; }
+}
+
 int ceil_log2(int n) { int b = 0; while ((1 << b) < n) ++b; return b; }
 
 size_t scan_lds_bytes(int E) { return sizeof(int32_t) * (size_t)(E + 2 * (E + 1) + 8); }
@@ -414,6 +452,28 @@ extern "C" int hexa_route_from_lists(const int32_t* token_idx_list, const int32_
         if (e1 != hipSuccess || e2 != hipSuccess) HEXA_FAIL(HEXA_ERR_LAUNCH, "hexa_route_from_lists: copy failed");
     }
     hipLaunchKernelGGL(route_from_lists_kernel, dim3(k), dim3(256), scan_lds_bytes(E), st, expert_idx_list, T, E,
+                       route + L.counts, route + L.offsets, reinterpret_cast<int4*>(route + L.tile_info),
+                       route + L.tile_count, L.mt_ub, reinterpret_cast<int4*>(route + L.tile_info_l),
+                       route + L.tile_count_l, L.mt_ub_l);
+    HEXA_CHECK_LAUNCH("route_from_lists");
+    return HEXA_OK;
+}
+
+extern "C" int hexa_route_from_padded_lists(const int32_t* token_idx_list, const int32_t* expert_idx_list,
+                                            const int32_t* slot_ends, int64_t list_len, int T, int k, int E,
+                                            int32_t* route, void* stream) {
+    if (int rc = check_route_sizes("hexa_route_from_padded_lists", T, k, E)) return rc;
+    if (!route || !slot_ends || list_len < 0 || (list_len > 0 && (!token_idx_list || !expert_idx_list)))
+        HEXA_FAIL(HEXA_ERR_ARG, "hexa_route_from_padded_lists: bad arguments");
+    if (((uintptr_t)route & 15) != 0)
+        HEXA_FAIL(HEXA_ERR_ARG, "hexa_route_from_padded_lists: route blob must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    hexa_route_layout L;
+    hexa_route_layout_get(T, k, E, &L);
+    hipLaunchKernelGGL(route_compact_kernel, dim3(k), dim3(1024), 0, st, token_idx_list, expert_idx_list, slot_ends,
+                       list_len, T, E, route + L.token_ids, route + L.expert_ids);
+    HEXA_CHECK_LAUNCH("route_compact");
+    hipLaunchKernelGGL(route_from_lists_kernel, dim3(k), dim3(256), scan_lds_bytes(E), st, route + L.expert_ids, T, E,
                        route + L.counts, route + L.offsets, reinterpret_cast<int4*>(route + L.tile_info),
                        route + L.tile_count, L.mt_ub, reinterpret_cast<int4*>(route + L.tile_info_l),
                        route + L.tile_count_l, L.mt_ub_l);

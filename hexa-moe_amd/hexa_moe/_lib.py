@@ -34,6 +34,7 @@ SIGNATURES = {
     "hexa_token_count": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "hexa_token_assign": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "hexa_route_from_lists": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
+    "hexa_route_from_padded_lists": (_i, [_vp, _vp, _vp, _i64, _i, _i, _i, _vp, _vp]),
     "hexa_esmm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "hexa_estmm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp]),
     "hexa_estmm_plan": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),

@@ -165,6 +165,20 @@ def route_from_lists(token_idx_list, expert_idx_list, T, k, num_experts, blob=No
     return Route(blob, T, k, num_experts)
 
 
+def route_from_padded_lists(token_idx_list, expert_idx_list, slot_ends, T, k, num_experts, blob=None):
+    """Route from the reference's concatenated, 16-padded lists; slot_ends is its device tensor of
+    k+1 cumulative list lengths (cum_ids of impls/layers.py:245-248)."""
+    _dev(token_idx_list, expert_idx_list, slot_ends)
+    if slot_ends.dtype != torch.int32 or slot_ends.numel() < k + 1 or not slot_ends.is_contiguous():
+        raise TypeError("slot_ends must be a contiguous int32 tensor of top_k + 1 entries")
+    if blob is None:
+        blob = torch.empty(max(route_blob_ints(T, k, num_experts), 4), dtype=torch.int32, device=token_idx_list.device)
+    rc = _lib.load().hexa_route_from_padded_lists(_ptr(token_idx_list), _ptr(expert_idx_list), _ptr(slot_ends),
+                                                  int(token_idx_list.numel()), T, k, num_experts, _ptr(blob), _stream())
+    _lib.check(rc, "hexa_route_from_padded_lists")
+    return Route(blob, T, k, num_experts)
+
+
 def esmm(x, w, bias, route, m2s, w_layout, out=None, out_dtype=None, accumulate=False, gelu=False, gelu_bwd_of=None):
     """out[(s),t] (+)= x[(s),t] @ W[e] + bias[e].  Returns out, or (out, gelu(out)) when gelu=True.
     gelu_bwd_of=y1 multiplies the result by gelu'(y1) (y1 of out's shape and dtype)."""

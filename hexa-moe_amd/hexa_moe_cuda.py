@@ -10,7 +10,8 @@ Differences that a caller can observe:
   * segments are not padded: expanded_tokens_per_expert is the exact exclusive prefix, so the lists
     the caller sizes from its last entry (impls/layers.py:238) have exactly num_tokens entries.
     set_pad(16) switches TOKEN_COUNT / TOKEN_ASSIGN to the reference's 16-padded format; the matmul
-    ops accept unpadded lists only.
+    ops take either format (padded lists are compacted on the device from num_expanded_tokens, the
+    cumulative list lengths, before the operators run).
   * the order inside a segment is ascending token id (the reference's depends on atomics).
   * element types come from the tensors; the *_dtype_full flags are checked against them.  bf16 is
     accepted wherever fp16 is.
@@ -65,12 +66,17 @@ def TOKEN_ASSIGN(token_idx_list, expert_idx_list, expanded_tokens_per_expert, ro
     _lib.check(rc, "TOKEN_ASSIGN")
 
 
-def _route(token_idx_list, expert_idx_list, num_tokens, top_k, num_routings):
+def _route(token_idx_list, expert_idx_list, num_expanded_tokens, num_tokens, top_k, num_routings):
     _i32(token_idx_list, "token_idx_list"); _i32(expert_idx_list, "expert_idx_list")
-    if token_idx_list.numel() != num_tokens * top_k or expert_idx_list.numel() != num_tokens * top_k:
-        raise NotImplementedError(
-            "the matmul operators take unpadded lists (top_k * num_tokens entries); build them with pad 1")
-    return ops.route_from_lists(token_idx_list, expert_idx_list, int(num_tokens), int(top_k), int(num_routings))
+    if token_idx_list.numel() != expert_idx_list.numel():
+        raise ValueError("token_idx_list and expert_idx_list differ in length")
+    if token_idx_list.numel() == num_tokens * top_k:     # exact lists: nothing to drop
+        return ops.route_from_lists(token_idx_list, expert_idx_list, int(num_tokens), int(top_k), int(num_routings))
+    if token_idx_list.numel() < num_tokens * top_k:
+        raise ValueError("the lists hold fewer than top_k * num_tokens entries")
+    _i32(num_expanded_tokens, "num_expanded_tokens")
+    return ops.route_from_padded_lists(token_idx_list, expert_idx_list, num_expanded_tokens, int(num_tokens),
+                                       int(top_k), int(num_routings))
 
 
 def _check_flag(t, full, what):
@@ -83,7 +89,7 @@ def ESMM_TENSOR_CORE(result, tokens, weights, bias, token_idx_list, expert_idx_l
                      num_routings):
     T, k, E = int(num_tokens), int(top_k), int(num_routings)
     _check_flag(tokens, x_dtype_full, "tokens"); _check_flag(weights, w_dtype_full, "weights")
-    route = _route(token_idx_list, expert_idx_list, T, k, E)
+    route = _route(token_idx_list, expert_idx_list, num_expanded_tokens, T, k, E)
     x = tokens.reshape((k, T, num_in_dims) if m2s else (T, num_in_dims))
     w = weights.reshape(E, num_in_dims, num_out_dims)
     b = bias.reshape(E, num_out_dims) if bias is not None and bias.numel() > 0 else None
@@ -92,10 +98,10 @@ def ESMM_TENSOR_CORE(result, tokens, weights, bias, token_idx_list, expert_idx_l
     ops.esmm(x, w, b, route, bool(m2s), _lib.HEXA_W_IN_OUT, out=out, accumulate=True)
 
 
-def _fused(j_b, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, m2s, num_tokens, top_k, num_in_dims,
-           num_out_dims, num_routings):
+def _fused(j_b, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, num_expanded_tokens, m2s, num_tokens, top_k,
+           num_in_dims, num_out_dims, num_routings):
     T, k, E = int(num_tokens), int(top_k), int(num_routings)
-    route = _route(token_idx_list, expert_idx_list, T, k, E)
+    route = _route(token_idx_list, expert_idx_list, num_expanded_tokens, T, k, E)
     for t in (j_x, j_w, j_y, w, x) + ((j_b,) if j_b is not None else ()):
         ops._dev(t)
         if not t.is_contiguous():
@@ -112,12 +118,12 @@ def _fused(j_b, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, m2s, num_t
 def FUSED_GRAD(j_b, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, num_expanded_tokens, x_dtype_full,
                w_dtype_full, m2s, num_tokens, top_k, num_in_dims, num_out_dims, num_routings):
     _check_flag(j_y, x_dtype_full, "j_y"); _check_flag(w, w_dtype_full, "w")
-    _fused(j_b, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, m2s, num_tokens, top_k, num_in_dims,
-           num_out_dims, num_routings)
+    _fused(j_b, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, num_expanded_tokens, m2s, num_tokens, top_k,
+           num_in_dims, num_out_dims, num_routings)
 
 
 def FUSED_GRAD_NO_BIAS(j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, num_expanded_tokens, x_dtype_full,
                        w_dtype_full, m2s, num_tokens, top_k, num_in_dims, num_out_dims, num_routings):
     _check_flag(j_y, x_dtype_full, "j_y"); _check_flag(w, w_dtype_full, "w")
-    _fused(None, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, m2s, num_tokens, top_k, num_in_dims,
-           num_out_dims, num_routings)
+    _fused(None, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, num_expanded_tokens, m2s, num_tokens, top_k,
+           num_in_dims, num_out_dims, num_routings)

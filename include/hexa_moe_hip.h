@@ -104,6 +104,16 @@ int hexa_token_assign(int32_t* token_idx_list, int32_t* expert_idx_list,
 int hexa_route_from_lists(const int32_t* token_idx_list, const int32_t* expert_idx_list, int num_tokens,
                           int top_k, int num_experts, int32_t* route, void* stream);
 
+/* The same from the reference's own list format: the k slots' lists concatenated, every expert's
+ * segment padded to a multiple of 16 with -1 (kernels/shared_cuda_core.cu:165-171 as called from
+ * impls/layers.py:233-249), slot s occupying [slot_ends[s], slot_ends[s+1]) of the lists; slot_ends
+ * is the caller's device array of k+1 cumulative lengths (cum_ids, impls/layers.py:245-248) and
+ * list_len the lists' total length.  Fillers are dropped in place of being skipped by every operator
+ * (kernels/esmm_full.cu:96-101); entries keep their order. */
+int hexa_route_from_padded_lists(const int32_t* token_idx_list, const int32_t* expert_idx_list,
+                                 const int32_t* slot_ends, int64_t list_len, int num_tokens, int top_k,
+                                 int num_experts, int32_t* route, void* stream);
+
 /* ESMM: out[(s),t,:] (+)= x[(s),t,:] . W[e_s(t)] + bias[e_s(t)] over all routed (slot, token) pairs.
  *   m2s == 0: x [T,in] shared by the slots, out [k,T,out]      (fc1 of the MoE FFN)
  *   m2s != 0: x [k,T,in] per slot,          out [T,out] = sum over slots (fc2; deterministic order)

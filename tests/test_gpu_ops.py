@@ -220,8 +220,20 @@ def test_esmm_fused_gelu_bwd(dev, dtype, d_in, d_out):
         assert_close(got, want, TOL[dtype], "esmm * gelu'")
 
 
-def test_reference_style_ops(dev):
-    """The five operator names of the reference extension, called the way impls/layers.py calls them."""
+@pytest.mark.parametrize("pad", [1, 16])
+def test_reference_style_ops(dev, pad):
+    """The five operator names of the reference extension, called the way impls/layers.py calls them:
+    with exact lists (pad 1) and with the reference's own format, every expert's segment padded to a
+    multiple of 16 with -1 and the slots' lists concatenated (pad 16)."""
+    import hexa_moe_cuda
+    hexa_moe_cuda.set_pad(pad)
+    try:
+        _reference_style_ops(dev, pad)
+    finally:
+        hexa_moe_cuda.set_pad(1)
+
+
+def _reference_style_ops(dev, pad):
     import hexa_moe_cuda
     T, d_in, d_out, E, k = 600, 64, 128, 8, 2
     routing = make_routing(T, E, k, seed=21).to(torch.int32)
@@ -239,6 +251,7 @@ def test_reference_style_ops(dev):
         tok_lists.append(torch.zeros(n, dtype=torch.int32, device=dev) - 1)
         exp_lists.append(torch.zeros(n, dtype=torch.int32, device=dev) - 1)
         hexa_moe_cuda.TOKEN_ASSIGN(tok_lists[i], exp_lists[i], expd, rd[:, i].contiguous(), T, E)
+        assert n % pad == 0 and (n > T) == (pad > 1) and int((tok_lists[i] >= 0).sum()) == T
     cum = torch.zeros(k + 1, dtype=torch.int32, device=dev)
     for i in range(k):
         cum[i + 1] = cum[i] + len(exp_lists[i])

@@ -112,3 +112,50 @@ def test_legacy_count_assign(dev, pad):
     assert np.array_equal(expd.cpu().numpy(), x_ref)
     assert np.array_equal(tok.cpu().numpy(), t_ref)
     assert np.array_equal(exp.cpu().numpy(), e_ref)
+
+
+@pytest.mark.parametrize("T,E,k,skew,empty", [(5000, 32, 2, "zipf", 3), (777, 5, 3, None, 0), (18432, 32, 2, None, 0)])
+def test_route_from_padded_lists(dev, T, E, k, skew, empty):
+    """The reference's list format (segments padded to 16 with -1, slots concatenated, cumulative
+    lengths in a device array) gives the same route as the routing decision itself.  The lists are
+    written by the C oracle; within a segment they are then permuted with a seeded shuffle, since the
+    reference's order inside a segment is whatever its atomics produced."""
+    from hexa_moe import ops
+    from oracle import route_oracle as RO
+    print(f"padded lists T={T} E={E} k={k} skew={skew}", flush=True)
+    routing = make_routing(T, E, k, seed=300 + T, skew=skew, empty=empty).to(torch.int32)
+    rng = np.random.default_rng(T)
+    toks, exps, ends = [], [], [0]
+    for s in range(k):
+        r = routing[:, s].contiguous().numpy()
+        _, x_ref = RO.token_count(r, E, 16)
+        t_ref, e_ref = RO.token_assign(r, E, x_ref)
+        toks.append(t_ref); exps.append(e_ref); ends.append(ends[-1] + len(t_ref))
+    tok = torch.from_numpy(np.concatenate(toks)).to(dev)
+    exp = torch.from_numpy(np.concatenate(exps)).to(dev)
+    cum = torch.tensor(ends, dtype=torch.int32, device=dev)
+    want = ops.route_build(routing.to(dev), E)
+    got = ops.route_from_padded_lists(tok, exp, cum, T, k, E)
+    torch.cuda.synchronize()
+    for name in ("counts", "offsets", "token_ids", "expert_ids", "tile_count", "tile_count_l"):
+        assert torch.equal(getattr(got, name), getattr(want, name)), name
+    for s in range(k):
+        n, nl = int(want.tile_count[s]), int(want.tile_count_l[s])
+        assert torch.equal(got.tile_info[s, :n], want.tile_info[s, :n])
+        assert torch.equal(got.tile_info_l[s, :nl], want.tile_info_l[s, :nl])
+    # shuffled inside each segment: same counts and offsets, each segment the same set of tokens
+    counts, offsets, _ = O.route_build(routing.long(), E)
+    shuf = [t.copy() for t in toks]
+    for s in range(k):
+        _, x_ref = RO.token_count(routing[:, s].contiguous().numpy(), E, 16)
+        for e in range(E):
+            a, c = int(x_ref[e]), int(counts[s, e])
+            rng.shuffle(shuf[s][a:a + c])
+    got2 = ops.route_from_padded_lists(torch.from_numpy(np.concatenate(shuf)).to(dev), exp, cum, T, k, E)
+    torch.cuda.synchronize()
+    assert torch.equal(got2.counts.cpu(), counts) and torch.equal(got2.offsets.cpu(), offsets)
+    ids = got2.token_ids.cpu()
+    for s in range(k):
+        for e in range(E):
+            a, b = int(offsets[s, e]), int(offsets[s, e + 1])
+            assert torch.equal(torch.sort(ids[s, a:b]).values, want.token_ids[s, a:b].cpu())

@@ -58,9 +58,14 @@ class MLP_Implement:
         return out
 
 
-def _weight_for(x, w):
-    """Kernels take weights in the tokens' 16-bit type or in fp32; anything else is converted."""
-    if w.dtype == x.dtype or (w.dtype == torch.float32 and x.dtype != torch.float32):
+def _weight_for(x, w, rows):
+    """Kernels take weights in the tokens' 16-bit type or in fp32.  fp32 master weights under 16-bit
+    tokens (autocast) are rounded to the tokens' type by the kernel as it stages them; with enough
+    routed rows per expert it is cheaper to round them once here -- same values, and the forward and
+    backward kernels then read half the bytes and take the fast path."""
+    if w.dtype == x.dtype:
+        return w
+    if w.dtype == torch.float32 and x.dtype != torch.float32 and rows < 128 * w.shape[0]:
         return w
     return w.to(x.dtype)
 
@@ -84,7 +89,7 @@ class FusedMoE_Shared_CudaCore(torch.autograd.Function):
         if any(ctx.needs_input_grad):
             config.route_pool.bind(config.stage, route)  # keep the slot until this call's backward is done
 
-        w1, w2 = _weight_for(x, fc1_w), _weight_for(x, fc2_w)
+        w1, w2 = _weight_for(x, fc1_w, T * routing.shape[1]), _weight_for(x, fc2_w, T * routing.shape[1])
         act = config.activation_fn
         fused = is_plain_gelu(act)
         ctx.act_graph = None

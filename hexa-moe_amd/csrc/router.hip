@@ -236,6 +236,182 @@ __global__ __launch_bounds__(ROUTER_TB) void router_bwd_kernel(float* __restrict
 }
 
 
+// ---- the same front end with the load-importance loss (impls/losses.py:21-42) ----------------------------
+// Per token: top-k of softmax(logits + noise_scale*noise) as above; thr = the k-th choice's noisy LOGIT;
+// s = softmax(logits) without noise; importance[e] += s[e]; load[e] += Phi((s[e] - thr) / sigma).  The
+// loss is the mean of the squared coefficients of variation (unbiased variance / (mean^2 + 1e-10)) of
+// importance and load.  One token per lane; the row (E floats) is walked in place, L1-resident.
+__device__ __forceinline__ float normal_cdf(float z) { return 0.5f * erfcf(-z * 0.70710678118654752f); }
+__device__ __forceinline__ float normal_pdf(float z) { return 0.3989422804014327f * expf(-0.5f * z * z); }
+
+__global__ __launch_bounds__(ROUTER_TB) void router_li_fwd_kernel(float* __restrict__ scores, int32_t* __restrict__ idx,
+                                                                  float* __restrict__ thr_out,
+                                                                  float* __restrict__ part_imp,
+                                                                  float* __restrict__ part_load,
+                                                                  const float* __restrict__ logits,
+                                                                  const float* __restrict__ noise, float noise_scale,
+                                                                  float inv_sigma, int num_tokens, int E, int k) {
+    const int lane = threadIdx.x;
+    const int t = blockIdx.x * ROUTER_TB + lane;
+    const bool ok = t < num_tokens;
+    const float* lr = logits + (size_t)(ok ? t : 0) * E;
+    const float* nr = noise ? noise + (size_t)(ok ? t : 0) * E : nullptr;
+    float best_v[MAX_TOPK];
+    int best_i[MAX_TOPK];
+#pragma unroll
+    for (int j = 0; j < MAX_TOPK; ++j) { best_v[j] = -INFINITY; best_i[j] = 0x7fffffff; }
+    // noisy scores: selection only
+    float mx = -INFINITY, cmx = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+        const float c = lr[e];
+        cmx = fmaxf(cmx, c);
+        mx = fmaxf(mx, nr ? c + noise_scale * nr[e] : c);
+    }
+    float sum = 0.f, csum = 0.f;
+    for (int e = 0; e < E; ++e) {
+        const float c = lr[e];
+        csum += expf(c - cmx);
+        sum += expf((nr ? c + noise_scale * nr[e] : c) - mx);
+    }
+    const float inv = 1.0f / sum, cinv = 1.0f / csum;
+    for (int e = 0; e < E; ++e) {
+        const float v = nr ? lr[e] + noise_scale * nr[e] : lr[e];
+        topk_insert(best_v, best_i, k, expf(v - mx) * inv, e);
+    }
+    int last = 0;
+#pragma unroll
+    for (int j = 0; j < MAX_TOPK; ++j)
+        if (j == k - 1) last = best_i[j];
+    float thr = 0.f;
+    if (ok) {
+        thr = nr ? lr[last] + noise_scale * nr[last] : lr[last];
+        thr_out[t] = thr;
+#pragma unroll
+        for (int j = 0; j < MAX_TOPK; ++j)
+            if (j < k) idx[(size_t)t * k + j] = best_i[j];
+    }
+    // clean scores, importance and load; uniform trip count: every lane takes part in the reductions
+    for (int e = 0; e < E; ++e) {
+        float sc = 0.f, ld = 0.f;
+        if (ok) {
+            sc = expf(lr[e] - cmx) * cinv;
+            scores[(size_t)t * E + e] = sc;
+            ld = normal_cdf((sc - thr) * inv_sigma);
+        }
+#pragma unroll
+        for (int m = 32; m > 0; m >>= 1) { sc += __shfl_xor(sc, m); ld += __shfl_xor(ld, m); }
+        if (lane == 0) {
+            part_imp[(size_t)blockIdx.x * E + e] = sc;
+            part_load[(size_t)blockIdx.x * E + e] = ld;
+        }
+    }
+}
+
+// importance / load from the workgroup partials (fixed order), the loss, and its derivative with
+// respect to each importance[e] and load[e] (kept for the backward pass):
+//   cv2(v) = var(v) / (mean(v)^2 + eps),  var unbiased;  d cv2 / d v[e] =
+//   2 (v[e] - mean) / ((E-1)(mean^2 + eps))  -  var * 2 mean / (E (mean^2 + eps)^2)
+// With a balanced router every v[e] is close to the mean, so v[e] - mean cancels almost all digits:
+// the sums over workgroups and everything after them are carried in double (one workgroup, a few
+// thousand operations).
+constexpr int ROUTER_LI_MAX_E = 1024;
+
+__global__ __launch_bounds__(256) void router_li_loss_kernel(float* __restrict__ l_aux, float* __restrict__ importance,
+                                                             float* __restrict__ load, float* __restrict__ g_imp,
+                                                             float* __restrict__ g_load,
+                                                             const float* __restrict__ part_imp,
+                                                             const float* __restrict__ part_load, int nblocks, int E) {
+    extern __shared__ double shd[];        // [nch][E] importance, [nch][E] load, then v_imp[E], v_load[E]
+    const int nch = max(1, min(32, 2048 / E));
+    double* s_a = shd;
+    double* s_b = shd + nch * E;
+    double* v_a = shd + 2 * nch * E;
+    double* v_b = v_a + E;
+    __shared__ double red[2][256];
+    const int per = (nblocks + nch - 1) / nch;
+    for (int i = threadIdx.x; i < nch * E; i += 256) {
+        const int c = i / E, e = i - c * E;
+        const int b0 = c * per, b1 = min(nblocks, b0 + per);
+        double a = 0., b = 0.;
+#pragma unroll 4
+        for (int q = b0; q < b1; ++q) { a += part_imp[(size_t)q * E + e]; b += part_load[(size_t)q * E + e]; }
+        s_a[i] = a;
+        s_b[i] = b;
+    }
+    __syncthreads();
+    double la = 0., lb = 0.;
+    for (int e = threadIdx.x; e < E; e += 256) {
+        double a = 0., b = 0.;
+        for (int j = 0; j < nch; ++j) { a += s_a[j * E + e]; b += s_b[j * E + e]; }
+        v_a[e] = a; v_b[e] = b;
+        importance[e] = (float)a; load[e] = (float)b;
+        la += a; lb += b;
+    }
+    auto block_sum2 = [&](double x, double y, double& ox, double& oy) {
+        red[0][threadIdx.x] = x; red[1][threadIdx.x] = y;
+        __syncthreads();
+        for (int s = 128; s > 0; s >>= 1) {
+            if (threadIdx.x < s) { red[0][threadIdx.x] += red[0][threadIdx.x + s]; red[1][threadIdx.x] += red[1][threadIdx.x + s]; }
+            __syncthreads();
+        }
+        ox = red[0][0]; oy = red[1][0];
+        __syncthreads();
+    };
+    double sa, sb;
+    block_sum2(la, lb, sa, sb);
+    const double ma = sa / E, mb = sb / E;
+    double qa = 0., qb = 0.;
+    for (int e = threadIdx.x; e < E; e += 256) {
+        const double da = v_a[e] - ma, db = v_b[e] - mb;
+        qa += da * da; qb += db * db;
+    }
+    double ssa, ssb;
+    block_sum2(qa, qb, ssa, ssb);
+    const double var_a = ssa / (E - 1), var_b = ssb / (E - 1);
+    const double den_a = ma * ma + 1e-10, den_b = mb * mb + 1e-10;
+    if (threadIdx.x == 0) *l_aux = (float)(0.5 * (var_a / den_a + var_b / den_b));
+    for (int e = threadIdx.x; e < E; e += 256) {
+        g_imp[e] = (float)(0.5 * (2. * (v_a[e] - ma) / ((E - 1) * den_a) - var_a * 2. * ma / (E * den_a * den_a)));
+        g_load[e] = (float)(0.5 * (2. * (v_b[e] - mb) / ((E - 1) * den_b) - var_b * 2. * mb / (E * den_b * den_b)));
+    }
+}
+
+// d l_aux / d logits:  ds[e] = g_imp[e] + g_load[e] * pdf(z[e]) / sigma,  z[e] = (s[e] - thr) / sigma;
+// through the noise-free softmax  dlogits[e] = s[e] (ds[e] - sum_e' s[e'] ds[e']);  and through the
+// threshold, which is the k-th choice's own logit:  dlogits[last] -= sum_e g_load[e] pdf(z[e]) / sigma.
+__global__ __launch_bounds__(ROUTER_TB) void router_li_bwd_kernel(float* __restrict__ dlogits,
+                                                                  const float* __restrict__ scores,
+                                                                  const float* __restrict__ thr,
+                                                                  const int32_t* __restrict__ idx,
+                                                                  const float* __restrict__ g_imp,
+                                                                  const float* __restrict__ g_load,
+                                                                  const float* __restrict__ grad_l, float inv_sigma,
+                                                                  int num_tokens, int E, int k) {
+    extern __shared__ float s_g[];         // g_imp[E], g_load[E] scaled by the incoming gradient
+    const float g = *grad_l;
+    for (int e = threadIdx.x; e < E; e += blockDim.x) { s_g[e] = g * g_imp[e]; s_g[E + e] = g * g_load[e] * inv_sigma; }
+    __syncthreads();
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= num_tokens) return;
+    const float* sr = scores + (size_t)t * E;
+    float* dr = dlogits + (size_t)t * E;
+    const float th = thr[t];
+    float dot = 0.f, dthr = 0.f;
+    for (int e = 0; e < E; ++e) {
+        const float sc = sr[e];
+        const float w = s_g[E + e] * normal_pdf((sc - th) * inv_sigma);
+        dot += sc * (s_g[e] + w);
+        dthr -= w;
+    }
+    const int last = idx[(size_t)t * k + (k - 1)];
+    for (int e = 0; e < E; ++e) {
+        const float sc = sr[e];
+        const float w = s_g[E + e] * normal_pdf((sc - th) * inv_sigma);
+        dr[e] = sc * (s_g[e] + w - dot) + (e == last ? dthr : 0.f);
+    }
+}
+
+
 }  // namespace
 }  // namespace hexa
 
@@ -280,5 +456,47 @@ extern "C" int hexa_router_backward(float* dlogits, const float* scores, const f
     hipLaunchKernelGGL(router_bwd_kernel, dim3(div_up(T, ROUTER_TB)), dim3(ROUTER_TB), sizeof(float) * E,
                        (hipStream_t)stream, dlogits, scores, ce, grad_l_aux, T, E);
     HEXA_CHECK_LAUNCH("router_bwd");
+    return HEXA_OK;
+}
+
+extern "C" int hexa_router_forward_load_importance(float* scores, int32_t* idx, float* thr, float* importance,
+                                                   float* load, float* g_importance, float* g_load, float* l_aux,
+                                                   const float* logits, const float* noise, float noise_scale,
+                                                   float sigma, int T, int E, int k, float* ws, void* stream) {
+    const char* who = "hexa_router_forward_load_importance";
+    if (T < 1 || E < 2 || k < 1) HEXA_FAIL(HEXA_ERR_ARG, "%s: bad sizes T=%d E=%d k=%d (E >= 2 for a variance)", who, T, E, k);
+    if (k > MAX_TOPK || k > E) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "%s: top_k must be <= min(E, %d)", who, MAX_TOPK);
+    if (!(sigma > 0.f)) HEXA_FAIL(HEXA_ERR_ARG, "%s: sigma must be > 0 (gate_noise / E of the reference)", who);
+    if (!scores || !idx || !thr || !importance || !load || !g_importance || !g_load || !l_aux || !logits || !ws)
+        HEXA_FAIL(HEXA_ERR_ARG, "%s: null pointer", who);
+    if (E > ROUTER_LI_MAX_E) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "%s: more than %d experts", who, ROUTER_LI_MAX_E);
+    hipStream_t st = (hipStream_t)stream;
+    const int nb = div_up(T, ROUTER_TB);
+    float* part_imp = ws;
+    float* part_load = ws + (size_t)nb * E;
+    hipLaunchKernelGGL(router_li_fwd_kernel, dim3(nb), dim3(ROUTER_TB), 0, st, scores, idx, thr, part_imp, part_load,
+                       logits, noise, noise_scale, 1.0f / sigma, T, E, k);
+    HEXA_CHECK_LAUNCH("router_li_fwd");
+    const int nch = std::max(1, std::min(32, 2048 / E));
+    hipLaunchKernelGGL(router_li_loss_kernel, dim3(1), dim3(256), sizeof(double) * (2 * nch * E + 2 * E), st, l_aux,
+                       importance, load, g_importance, g_load, part_imp, part_load, nb, E);
+    HEXA_CHECK_LAUNCH("router_li_loss");
+    return HEXA_OK;
+}
+
+extern "C" int hexa_router_backward_load_importance(float* dlogits, const float* scores, const float* thr,
+                                                    const int32_t* idx, const float* g_importance,
+                                                    const float* g_load, const float* grad_l_aux, float sigma, int T,
+                                                    int E, int k, void* stream) {
+    const char* who = "hexa_router_backward_load_importance";
+    if (T < 1 || E < 2 || k < 1 || k > E) HEXA_FAIL(HEXA_ERR_ARG, "%s: bad sizes", who);
+    if (!(sigma > 0.f)) HEXA_FAIL(HEXA_ERR_ARG, "%s: sigma must be > 0", who);
+    if (!dlogits || !scores || !thr || !idx || !g_importance || !g_load || !grad_l_aux)
+        HEXA_FAIL(HEXA_ERR_ARG, "%s: null pointer", who);
+    if (E > 4096) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "%s: more than 4096 experts", who);
+    hipLaunchKernelGGL(router_li_bwd_kernel, dim3(div_up(T, ROUTER_TB)), dim3(ROUTER_TB), sizeof(float) * 2 * E,
+                       (hipStream_t)stream, dlogits, scores, thr, idx, g_importance, g_load, grad_l_aux, 1.0f / sigma,
+                       T, E, k);
+    HEXA_CHECK_LAUNCH("router_li_bwd");
     return HEXA_OK;
 }

@@ -47,6 +47,9 @@ SIGNATURES = {
     "hexa_router_ws_floats": (_i, [_i, _i, ctypes.POINTER(_i64)]),
     "hexa_router_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float, _i, _i, _i, _vp, _vp]),
     "hexa_router_backward": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "hexa_router_forward_load_importance": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float,
+                                                 ctypes.c_float, _i, _i, _i, _vp, _vp]),
+    "hexa_router_backward_load_importance": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float, _i, _i, _i, _vp]),
     "hexa_last_error": (ctypes.c_char_p, []),
     "hexa_abi_version": (_i, []),
     "hexa_set_option": (_i, [ctypes.c_char_p, _i]),
@@ -69,7 +72,7 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.hexa_abi_version() != 4:
+    if lib.hexa_abi_version() != 5:
         raise RuntimeError("hexa_moe: libhexa_moe_hip.so has an unexpected ABI version")
     _lib = lib
     return lib

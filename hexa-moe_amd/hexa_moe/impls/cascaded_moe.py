@@ -264,11 +264,11 @@ class MoE_Cascaded(nn.Module):
     # ---- forward -----------------------------------------------------------------------------------
     def _route(self, gate, x, top_k):
         """gate -> (+noise) -> softmax -> top-k and the auxiliary loss (reference: cascaded_moe.py:515-531).
-        GPU inputs with the linear gate and the GShard loss take the fused kernels (impls/router.py)."""
+        GPU inputs with the linear gate take the fused kernels (impls/router.py)."""
         if self.fused_router and router.fused_route_supported(gate, x, top_k, self.num_global_experts,
                                                               self.is_gshard_loss):
             return router.fused_route(gate, x, top_k, self.num_global_experts,
-                                      gate.gate_noise / self.num_global_experts, self.training)
+                                      gate.gate_noise / self.num_global_experts, self.training, self.is_gshard_loss)
         logits = gate(x)
         if self.training and gate.gate_noise > 0:
             logits_w_noise = logits + gate.gate_noise * torch.randn_like(logits) / self.num_global_experts

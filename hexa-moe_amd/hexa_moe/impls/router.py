@@ -1,8 +1,8 @@
-"""Fused routing front end: gate projection, softmax, top-k and the GShard loss as HIP kernels with
-autograd glue.  It computes what the reference's routing() closure computes
-(hexa_moe_cuda/hexa_moe/impls/cascaded_moe.py:515-531 with impls/layers.py:476-484 and
-impls/losses.py:12-19); MoE_Cascaded uses it for GPU inputs with the linear gate and the GShard loss and
-keeps the PyTorch formulation for everything else (cosine gate, load-importance loss, more than 8 slots).
+"""Fused routing front end: gate projection, softmax, top-k and the auxiliary loss (GShard or
+load-importance) as HIP kernels with autograd glue.  It computes what the reference's routing() closure
+computes (hexa_moe_cuda/hexa_moe/impls/cascaded_moe.py:515-531 with impls/layers.py:476-484 and
+impls/losses.py:12-42); MoE_Cascaded uses it for GPU inputs with the linear gate and keeps the PyTorch
+formulation for everything else (cosine gate, more than 8 slots, a single expert).
 """
 import torch
 
@@ -43,14 +43,33 @@ class RouterTopK(torch.autograd.Function):
         return ops.router_backward(scores, ce, dl_aux), None, None, None
 
 
+class RouterTopKLoadImportance(torch.autograd.Function):
+    """(idx [T,k] int32, l_aux) with the load-importance loss; sigma = gate_noise / E."""
+
+    @staticmethod
+    def forward(ctx, logits, noise, noise_scale, sigma, top_k):
+        scores, idx, thr, stats = ops.router_forward_load_importance(logits, top_k, sigma, noise, noise_scale)
+        ctx.save_for_backward(scores, idx, thr, stats)
+        ctx.sigma = sigma
+        ctx.mark_non_differentiable(idx)
+        return idx, stats[-1]
+
+    @staticmethod
+    def backward(ctx, _didx, dl_aux):
+        scores, idx, thr, stats = ctx.saved_tensors
+        return ops.router_backward_load_importance(scores, thr, idx, stats, dl_aux, ctx.sigma), None, None, None, None
+
+
 def fused_route_supported(gate, x, top_k, num_experts, is_gshard_loss):
     from ..gates.top import LinearTopKGate
-    return (x.is_cuda and is_gshard_loss and isinstance(gate, LinearTopKGate) and 1 <= top_k <= min(8, num_experts)
+    if not is_gshard_loss and not (2 <= num_experts <= 1024 and gate.gate_noise > 0):
+        return False      # the PyTorch formulation raises the reference's error / yields its NaN
+    return (x.is_cuda and isinstance(gate, LinearTopKGate) and 1 <= top_k <= min(8, num_experts)
             and num_experts <= 4096 and x.shape[1] % 8 == 0
             and x.dtype in (torch.float32, torch.float16, torch.bfloat16))
 
 
-def fused_route(gate, x, top_k, num_experts, noise_scale, training):
+def fused_route(gate, x, top_k, num_experts, noise_scale, training, is_gshard_loss=True):
     """Returns (indices [T,k] int32, l_aux)."""
     w = gate.wg.weight
     if gate.fp32_gate or x.dtype == torch.float32:
@@ -60,4 +79,7 @@ def fused_route(gate, x, top_k, num_experts, noise_scale, training):
     noise = None
     if training and noise_scale > 0:
         noise = torch.randn_like(logits)
+    if not is_gshard_loss:
+        return RouterTopKLoadImportance.apply(logits, noise, float(noise_scale), float(gate.gate_noise) / num_experts,
+                                              int(top_k))
     return RouterTopK.apply(logits, noise, float(noise_scale), int(top_k))

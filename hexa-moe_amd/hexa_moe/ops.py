@@ -352,3 +352,41 @@ def router_backward(scores, ce, grad_l_aux):
                _stream())
     _lib.check(rc, "hexa_router_backward")
     return dlogits
+
+
+def router_forward_load_importance(logits, top_k, sigma, noise=None, noise_scale=0.0):
+    """softmax + top-k + load-importance loss.  Returns scores (noise-free softmax) [T,E] fp32, idx [T,k]
+    int32, thr [T], stats [4E+1] = importance, load, d l_aux/d importance, d l_aux/d load, l_aux."""
+    import ctypes
+    _dev(logits, noise)
+    logits = logits.contiguous()
+    assert logits.dtype == torch.float32 and logits.dim() == 2
+    T, E = logits.shape
+    dev = logits.device
+    n = ctypes.c_int64()
+    _lib.check(_lib.load().hexa_router_ws_floats(T, E, ctypes.byref(n)), "hexa_router_ws_floats")
+    ws = torch.empty(int(n.value), dtype=torch.float32, device=dev)
+    scores = torch.empty(T, E, dtype=torch.float32, device=dev)
+    idx = torch.empty(T, top_k, dtype=torch.int32, device=dev)
+    thr = torch.empty(T, dtype=torch.float32, device=dev)
+    stats = torch.empty(4 * E + 1, dtype=torch.float32, device=dev)
+    part = [stats[i * E:(i + 1) * E] for i in range(4)]
+    if noise is not None:
+        noise = noise.contiguous()
+        assert noise.dtype == torch.float32 and noise.shape == logits.shape
+    rc = _call("router_forward", _lib.load().hexa_router_forward_load_importance, _ptr(scores), _ptr(idx), _ptr(thr),
+               _ptr(part[0]), _ptr(part[1]), _ptr(part[2]), _ptr(part[3]), stats[4 * E].data_ptr(), _ptr(logits),
+               _ptr(noise), float(noise_scale), float(sigma), T, E, int(top_k), _ptr(ws), _stream())
+    _lib.check(rc, "hexa_router_forward_load_importance")
+    return scores, idx, thr, stats
+
+
+def router_backward_load_importance(scores, thr, idx, stats, grad_l_aux, sigma):
+    T, E = scores.shape
+    grad_l_aux = grad_l_aux.to(torch.float32).contiguous()
+    dlogits = torch.empty_like(scores)
+    rc = _call("router_backward", _lib.load().hexa_router_backward_load_importance, _ptr(dlogits), _ptr(scores),
+               _ptr(thr), _ptr(idx), _ptr(stats[2 * E:3 * E]), _ptr(stats[3 * E:4 * E]), _ptr(grad_l_aux), float(sigma),
+               T, E, int(idx.shape[1]), _stream())
+    _lib.check(rc, "hexa_router_backward_load_importance")
+    return dlogits

@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define HEXA_ABI_VERSION 4
+#define HEXA_ABI_VERSION 5
 
 /* element types */
 #define HEXA_F32 0
@@ -214,6 +214,25 @@ int hexa_router_forward(float* scores, int32_t* idx, float* me, float* ce, float
  * in the reference where the one-hot mask carries no gradient). */
 int hexa_router_backward(float* dlogits, const float* scores, const float* ce, const float* grad_l_aux,
                          int num_tokens, int num_experts, void* stream);
+
+/* The same front end with the load-importance loss of impls/losses.py:21-42 (what the Swin-MoE configs
+ * train with: IS_GSHARD_LOSS False).  idx = top-k of softmax(logits + noise_scale*noise); thr[t] = the
+ * k-th choice's noisy logit; scores = softmax(logits) WITHOUT noise; importance[e] = sum_t scores;
+ * load[e] = sum_t Phi((scores[t][e] - thr[t]) / sigma); l_aux = (cv2(importance) + cv2(load)) / 2 with
+ * cv2(v) = unbiased var / (mean^2 + 1e-10).  sigma is the reference's gate_noise / E (it divides by
+ * it whether or not noise was added).  g_importance / g_load [E] receive d l_aux / d importance, load
+ * for the backward call, which returns dlogits = d l_aux / d logits * (*grad_l_aux) through the
+ * softmax and through the threshold.  ws: hexa_router_ws_floats() floats.  2 <= E <= 1024.  The
+ * reductions over tokens and the variance are carried in double (v[e] - mean cancels).
+ * Replaces routing() + simplified_extract_critical + load_importance_loss
+ * (impls/cascaded_moe.py:515-531, impls/layers.py:476-484, impls/losses.py:21-42). */
+int hexa_router_forward_load_importance(float* scores, int32_t* idx, float* thr, float* importance, float* load,
+                                        float* g_importance, float* g_load, float* l_aux, const float* logits,
+                                        const float* noise, float noise_scale, float sigma, int num_tokens,
+                                        int num_experts, int top_k, float* ws, void* stream);
+int hexa_router_backward_load_importance(float* dlogits, const float* scores, const float* thr, const int32_t* idx,
+                                         const float* g_importance, const float* g_load, const float* grad_l_aux,
+                                         float sigma, int num_tokens, int num_experts, int top_k, void* stream);
 
 const char* hexa_last_error(void);
 int hexa_abi_version(void);

@@ -75,6 +75,52 @@ def test_router_forward_and_backward(dev, T, E, k, with_noise):
     assert_close(got, want, 1e-5, "dlogits")
 
 
+def _load_importance_fp64(logits, noisy, idx, sigma):
+    """The loss in double precision, differentiable with respect to `logits` (noisy = logits + noise)."""
+    s = F.softmax(logits, dim=1)
+    thr = noisy.gather(1, idx[:, -1:])
+    load = torch.special.ndtr((s - thr) / sigma).sum(0)
+    imp = s.sum(0)
+    return (imp.var() / (imp.mean() ** 2 + 1e-10) + load.var() / (load.mean() ** 2 + 1e-10)) / 2
+
+
+@pytest.mark.parametrize("T,E,k", [(1000, 32, 1), (9216, 32, 1), (18432, 32, 2), (2048, 8, 2), (513, 70, 3), (64, 4, 4)])
+@pytest.mark.parametrize("with_noise", [False, True])
+@pytest.mark.parametrize("spread", [0.02, 1.0])
+def test_router_load_importance(dev, T, E, k, with_noise, spread):
+    """softmax + top-k + the load-importance loss and its backward against the PyTorch formulation:
+    identical expert choices, loss against the oracle, gradient against fp64 autograd.  spread 0.02 is
+    the regime of a freshly initialised gate (scores near 1/E, thresholds near 0: the normal CDF is in
+    its steep part), spread 1.0 that of a trained one (saturated CDF)."""
+    from hexa_moe import ops
+    g = gen(T * k + E + 7)
+    logits = spread * (torch.randn(T, E, generator=g) + 0.5 * torch.randn(E, generator=g))
+    noise = torch.randn(T, E, generator=g) if with_noise else None
+    gate_noise = 1.0
+    sigma = gate_noise / E
+    noisy = logits + noise * sigma if with_noise else logits
+    _, idx_ref = O.route_top_k(noisy, k)
+    want_l = O.load_importance_loss(F.softmax(logits, 1), noisy.gather(1, idx_ref), E, gate_noise)
+    scores, idx, thr, stats = ops.router_forward_load_importance(logits.to(dev), k, sigma,
+                                                                 noise.to(dev) if with_noise else None, sigma)
+    torch.cuda.synchronize()
+    assert torch.equal(idx.cpu().long(), idx_ref)
+    assert_close(scores, F.softmax(logits.double(), 1), 1e-6, "scores")
+    assert_close(thr, noisy.gather(1, idx_ref[:, -1:]).reshape(-1), 1e-6, "threshold")
+    imp, load, l_aux = stats[:E], stats[E:2 * E], stats[4 * E]
+    assert_close(imp, F.softmax(logits.double(), 1).sum(0), 1e-5, "importance")
+    z = (F.softmax(logits.double(), 1) - noisy.double().gather(1, idx_ref[:, -1:])) / sigma
+    assert_close(load, torch.special.ndtr(z).sum(0), 1e-4, "load")
+    assert_close(l_aux.reshape(1), want_l.reshape(1).double(), 1e-3, "l_aux vs oracle (fp32)")
+    lg = logits.double().requires_grad_(True)
+    l64 = _load_importance_fp64(lg, lg + (noise.double() * sigma if with_noise else 0), idx_ref, sigma)
+    assert_close(l_aux.reshape(1), l64.detach().reshape(1), 1e-4, "l_aux vs fp64")
+    (want_g,) = torch.autograd.grad(l64 * 3.0, lg)
+    got_g = ops.router_backward_load_importance(scores, thr, idx, stats, torch.tensor(3.0, device=dev), sigma)
+    torch.cuda.synchronize()
+    assert_close(got_g, want_g, 1e-4, "dlogits")
+
+
 def test_ties_go_to_the_lower_index(dev):
     from hexa_moe import ops
     logits = torch.zeros(5, 6)
@@ -84,15 +130,21 @@ def test_ties_go_to_the_lower_index(dev):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_module_fused_and_framework_routing_agree(dev, dtype):
+@pytest.mark.parametrize("gshard", [True, False])
+def test_module_fused_and_framework_routing_agree(dev, dtype, gshard):
+    """MoE_Cascaded with the fused routing front end and with the PyTorch formulation of it.  The
+    load-importance case runs in eval mode: it needs gate_noise > 0 for its sigma, and only without
+    drawn noise do the two runs see the same logits."""
     from hexa_moe import moe as hmoe
     torch.manual_seed(3)
-    m = hmoe.MoE_Cascaded(gate_type={'type': 'top', 'k': 2, 'gate_noise': 0.0, 'fp32_gate': True}, model_dim_list=[256],
-                          moe_idx_list=[0], num_global_experts=16, total_depth=1, data_centric=True,
-                          activation_fn=F.gelu)
+    m = hmoe.MoE_Cascaded(gate_type={'type': 'top', 'k': 2, 'gate_noise': 0.0 if gshard else 1.0, 'fp32_gate': True},
+                          model_dim_list=[256], moe_idx_list=[0], num_global_experts=16, total_depth=1,
+                          data_centric=True, activation_fn=F.gelu, is_gshard_loss=gshard)
     for p in m.parameters():
         torch.nn.init.uniform_(p.data, -0.06, 0.06)
     m = m.to(dev)
+    if not gshard:
+        m.eval()
     if dtype != torch.float32:
         m = m.to(dtype)
     x = torch.randn(3000, 256, device=dev).to(dtype)

@@ -60,12 +60,14 @@ class MLP_Implement:
 
 def _weight_for(x, w, rows):
     """Kernels take weights in the tokens' 16-bit type or in fp32.  fp32 master weights under 16-bit
-    tokens (autocast) are rounded to the tokens' type by the kernel as it stages them; with enough
-    routed rows per expert it is cheaper to round them once here -- same values, and the forward and
-    backward kernels then read half the bytes and take the fast path."""
+    tokens (autocast) are rounded to the tokens' type by the kernel as it stages them; from a few dozen
+    routed rows per expert on it is cheaper to round them once here -- same values, and the forward and
+    backward kernels then read half the bytes and take the fast path (measured at 72 rows per expert,
+    768 -> 3072, 32 experts: forward + backward ESMM 218 + 188 us on fp32 weights, 72 + 60 us on the
+    rounded copy, whose making moves 450 MB once)."""
     if w.dtype == x.dtype:
         return w
-    if w.dtype == torch.float32 and x.dtype != torch.float32 and rows < 128 * w.shape[0]:
+    if w.dtype == torch.float32 and x.dtype != torch.float32 and rows < 32 * w.shape[0]:
         return w
     return w.to(x.dtype)
 

@@ -35,10 +35,13 @@ class RouterTopK(torch.autograd.Function):
         scores, idx, _me, ce, l_aux = ops.router_forward(logits, top_k, noise, noise_scale)
         ctx.save_for_backward(scores, ce)
         ctx.mark_non_differentiable(idx)
+        ctx.set_materialize_grads(False)    # no zero tensor for the index output's absent gradient
         return idx, l_aux
 
     @staticmethod
     def backward(ctx, _didx, dl_aux):
+        if dl_aux is None:
+            return None, None, None, None
         scores, ce = ctx.saved_tensors
         return ops.router_backward(scores, ce, dl_aux), None, None, None
 
@@ -52,10 +55,13 @@ class RouterTopKLoadImportance(torch.autograd.Function):
         ctx.save_for_backward(scores, idx, thr, stats)
         ctx.sigma = sigma
         ctx.mark_non_differentiable(idx)
+        ctx.set_materialize_grads(False)
         return idx, stats[-1]
 
     @staticmethod
     def backward(ctx, _didx, dl_aux):
+        if dl_aux is None:
+            return None, None, None, None, None
         scores, idx, thr, stats = ctx.saved_tensors
         return ops.router_backward_load_importance(scores, thr, idx, stats, dl_aux, ctx.sigma), None, None, None, None
 

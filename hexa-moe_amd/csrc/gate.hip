@@ -134,12 +134,12 @@ __global__ __launch_bounds__(256) void gate_fwd_kernel(float* __restrict__ logit
 
 // ---- dx: 32 tokens per workgroup, 128-column groups of the model dimension over the wavefronts ------
 template <typename T>
-__global__ __launch_bounds__(256) void gate_dx_kernel(T* __restrict__ dx, const float* __restrict__ dl,
-                                                      const float* __restrict__ wg, int num_tokens, int d, int E) {
+__device__ __forceinline__ void gate_dx_body(int block, T* __restrict__ dx, const float* __restrict__ dl,
+                                             const float* __restrict__ wg, int num_tokens, int d, int E) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, h = lane >> 5;
-    const int t0 = blockIdx.x * GT;
+    const int t0 = block * GT;
     const bool tok_ok = t0 + r < num_tokens;
     const float* drow = dl + (size_t)(t0 + r) * E;
     for (int g = wave; g * 128 < d; g += 4) {
@@ -187,15 +187,16 @@ __global__ __launch_bounds__(256) void gate_dx_kernel(T* __restrict__ dx, const 
 
 // ---- dwg: partial sums over DWG_TB tokens per workgroup, then a reduction in workgroup order ---------
 template <typename T>
-__global__ __launch_bounds__(256) void gate_dwg_kernel(float* __restrict__ part, const float* __restrict__ dl,
-                                                       const T* __restrict__ x, int num_tokens, int d, int E) {
+__device__ __forceinline__ void gate_dwg_body(int part_idx, int e_block, float* __restrict__ part,
+                                              const float* __restrict__ dl, const T* __restrict__ x, int num_tokens,
+                                              int d, int E) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, h = lane >> 5;
-    const int t0 = blockIdx.x * DWG_TB;
-    const int e0 = blockIdx.y * 32;
+    const int t0 = part_idx * DWG_TB;
+    const int e0 = e_block * 32;
     const bool exp_ok = e0 + r < E;
-    float* out = part + (size_t)blockIdx.x * E * d;
+    float* out = part + (size_t)part_idx * E * d;
     for (int g = wave; g * 128 < d; g += 4) {
         const int col = g * 128 + 4 * r;
         const bool col_ok = col < d;
@@ -222,6 +223,35 @@ __global__ __launch_bounds__(256) void gate_dwg_kernel(float* __restrict__ part,
                 if (e < E) store4<float>(out + (size_t)e * d + col, acc[0][v], acc[1][v], acc[2][v], acc[3][v]);
             }
         }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gate_dx_kernel(T* __restrict__ dx, const float* __restrict__ dl,
+                                                      const float* __restrict__ wg, int num_tokens, int d, int E) {
+    gate_dx_body<T>(blockIdx.x, dx, dl, wg, num_tokens, d, E);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gate_dwg_kernel(float* __restrict__ part, const float* __restrict__ dl,
+                                                       const T* __restrict__ x, int num_tokens, int d, int E) {
+    gate_dwg_body<T>(blockIdx.x, blockIdx.y, part, dl, x, num_tokens, d, E);
+}
+
+// Both products in one launch: each of them alone leaves most of the chip waiting on memory latency, and they
+// share nothing but their inputs.  Workgroups alternate (two dx workgroups per dwg workgroup of the same 64
+// tokens, so the dlogits rows they both read are fetched once).
+template <typename T>
+__global__ __launch_bounds__(256) void gate_bwd_kernel(T* __restrict__ dx, float* __restrict__ part,
+                                                       const float* __restrict__ dl, const T* __restrict__ x,
+                                                       const float* __restrict__ wg, int num_tokens, int d, int E,
+                                                       int e_blocks) {
+    const int per = 2 + e_blocks;                 // workgroups per 64 tokens
+    const int grp = blockIdx.x / per, role = blockIdx.x - grp * per;
+    if (role < 2) {
+        if ((2 * grp + role) * GT < num_tokens) gate_dx_body<T>(2 * grp + role, dx, dl, wg, num_tokens, d, E);
+    } else {
+        gate_dwg_body<T>(grp, role - 2, part, dl, x, num_tokens, d, E);
     }
 }
 
@@ -254,14 +284,22 @@ __global__ __launch_bounds__(256) void gate_dwg_reduce_kernel(float* __restrict_
 template <typename T>
 int gate_backward_t(void* dx, float* dwg, const float* dl, const void* x, const float* wg, int T_, int d, int E, float* ws,
                     hipStream_t st) {
-    if (dx) {
+    static_assert(DWG_TB == 2 * GT, "gate_bwd_kernel pairs two dx workgroups with one dwg workgroup");
+    if (dx && dwg) {
+        const int nparts = div_up(T_, DWG_TB), eb = div_up(E, 32);
+        hipLaunchKernelGGL(gate_bwd_kernel<T>, dim3(nparts * (2 + eb)), dim3(256), 0, st, (T*)dx, ws, dl, (const T*)x, wg,
+                           T_, d, E, eb);
+        HEXA_CHECK_LAUNCH("gate_bwd");
+    } else if (dx) {
         hipLaunchKernelGGL(gate_dx_kernel<T>, dim3(div_up(T_, GT)), dim3(256), 0, st, (T*)dx, dl, wg, T_, d, E);
         HEXA_CHECK_LAUNCH("gate_dx");
     }
     if (dwg) {
         const int nparts = div_up(T_, DWG_TB);
-        hipLaunchKernelGGL(gate_dwg_kernel<T>, dim3(nparts, div_up(E, 32)), dim3(256), 0, st, ws, dl, (const T*)x, T_, d, E);
-        HEXA_CHECK_LAUNCH("gate_dwg");
+        if (!dx) {
+            hipLaunchKernelGGL(gate_dwg_kernel<T>, dim3(nparts, div_up(E, 32)), dim3(256), 0, st, ws, dl, (const T*)x, T_, d, E);
+            HEXA_CHECK_LAUNCH("gate_dwg");
+        }
         const long n4 = (long)E * d / 4;
         hipLaunchKernelGGL(gate_dwg_reduce_kernel, dim3((unsigned)div_up(n4, 16)), dim3(256), 0, st, dwg, ws, nparts, n4);
         HEXA_CHECK_LAUNCH("gate_dwg_reduce");

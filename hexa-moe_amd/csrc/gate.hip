@@ -107,7 +107,6 @@ __global__ __launch_bounds__(256) void gate_fwd_kernel(float* __restrict__ logit
         const bool exp_ok = e0 + r < E;
         const float* wrow = wg + (size_t)(e0 + r) * d;
         f32x16 acc = zero16();
-#pragma unroll 2
         for (int c = c0; c < c1; ++c) {
             const int piece = 2 * c + h;
             const bool ok = piece < pieces;

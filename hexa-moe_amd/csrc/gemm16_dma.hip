@@ -618,6 +618,9 @@ int launch_estmm_dma_c(const EstmmArgs& a, hipStream_t st) {
     p.p_slot_rows = a.p_per_slot ? a.r.T : 0;
     p.q_slot_rows = a.q_per_slot ? a.r.T : 0;
     p.accumulate = a.accumulate;
+    // Runs of `group` tiles per XCD.  One row tile (with all its column tiles) per run is the fastest measured;
+    // 4 row tiles per run cut the launch's HBM fetch from 345 to 204 MB at the benchmark shape (the Q rows of an
+    // expert are then fetched by 3 of the 8 L2s instead of all of them) and cost 2 % in time.
     p.group = p.ntn * std::max(1, option(OPT_ESTMM_GROUP));
     p.plan = nullptr; p.scratch = nullptr;
     int units = a.r.E;
@@ -670,7 +673,9 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
         p.accumulate = (a.accumulate || l > 0) ? 1 : 0;
         p.total = (long)p.nslots * p.mt_ub * p.ntn;
         if (p.total == 0) continue;
-        const bool contiguous = p.nslots <= 8 && option(OPT_ESMM_MAP) == 1;
+        // default: every XCD walks one contiguous eighth of the valid tiles (least re-fetching of weights and
+        // token rows by several L2s); 2 selects runs of `group` tiles per XCD
+        const bool contiguous = p.nslots <= 8 && option(OPT_ESMM_MAP) != 2;
         const int grid = round_up(p.total, contiguous ? 8 : 8 * p.group);
         if (contiguous) p.group = 0;
         const bool io = a.w_layout == HEXA_W_IN_OUT;

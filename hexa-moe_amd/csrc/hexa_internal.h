@@ -81,7 +81,7 @@ enum Opt {
     OPT_TILE,           // HEXA_MOE_TILE: tile configuration of the 16-bit fast path (see gemm16_dma.hip)
     OPT_PERSIST,        // HEXA_MOE_PERSIST: 1 = persistent-workgroup ESMM kernels
     OPT_GENERAL,        // HEXA_MOE_GENERAL_KERNELS: 1 = general 16-bit kernels instead of the fast path
-    OPT_ESMM_MAP,       // HEXA_ESMM_MAP: 1 = every XCD walks one contiguous eighth of the tiles
+    OPT_ESMM_MAP,       // HEXA_ESMM_MAP: 2 = runs of tiles per XCD instead of one contiguous eighth of the tiles per XCD
     OPT_ESMM_GROUP,     // HEXA_ESMM_GROUP: row tiles per XCD run
     OPT_ESTMM_GROUP,    // HEXA_ESTMM_GROUP: row tiles per XCD run
     OPT_ESMM_STREAM,    // HEXA_ESMM_STREAM: 1 = results stored with the streaming hint

@@ -85,6 +85,7 @@ enum Opt {
     OPT_ESMM_GROUP,     // HEXA_ESMM_GROUP: row tiles per XCD run
     OPT_ESTMM_GROUP,    // HEXA_ESTMM_GROUP: row tiles per XCD run
     OPT_ESMM_STREAM,    // HEXA_ESMM_STREAM: 1 = results stored with the streaming hint
+    OPT_ROUTE_KERNELS,  // HEXA_ROUTE_KERNELS: 3 = always the three-launch routing pass, 1 = one launch up to 65536 tokens
     OPT_COUNT
 };
 int option(int id);

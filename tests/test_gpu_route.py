@@ -21,14 +21,27 @@ CASES = [
     (32768, 64, 2, "zipf", 4),
     (1000, 16, 2, "one", 0),
     (3000, 300, 2, None, 0),
+    (70000, 16, 2, None, 0),
+    (65536, 256, 1, "zipf", 20),
 ]
+
+
+@pytest.fixture(params=[1, 3], ids=["one_launch", "three_launches"])
+def route_kernels(request):
+    """The pass runs as one launch for small token counts, else as three; both are forced in turn on every
+    case (one launch covers up to 65536 tokens and 256 experts; beyond that it is three in both runs)."""
+    from hexa_moe import _lib
+    lib = _lib.load()
+    _lib.check(lib.hexa_set_option(b"route_kernels", request.param), "hexa_set_option")
+    yield request.param
+    _lib.check(lib.hexa_set_option(b"route_kernels", 0), "hexa_set_option")
 
 
 @pytest.mark.parametrize("T,E,k,skew,empty", CASES)
 @pytest.mark.parametrize("as_i64", [False, True])
-def test_route_build_matches_oracle(dev, T, E, k, skew, empty, as_i64):
+def test_route_build_matches_oracle(dev, route_kernels, T, E, k, skew, empty, as_i64):
     from hexa_moe import ops
-    print(f"case T={T} E={E} k={k} skew={skew} i64={as_i64}", flush=True)
+    print(f"case T={T} E={E} k={k} skew={skew} i64={as_i64} route_kernels={route_kernels}", flush=True)
     routing = make_routing(T, E, k, seed=100 + T + E, skew=skew, empty=empty)
     counts, offsets, token_ids = O.route_build(routing, E)
     r = routing if as_i64 else routing.to(torch.int32)

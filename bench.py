@@ -35,7 +35,7 @@ MEASURED_TRAFFIC_BYTES = {
     "estmm[1536x384]": 408.8e6 + 40.1e6,            # main kernel + the fixup of the experts cut into parts
     "esmm[1536->384,w_in_out,sum_slots]": 234.4e6 + 42.5e6,   # + the slot sum
     "esmm[384->1536,w_out_in,gelu]": 354.0e6,       # average over the two launches of this kernel
-    "esmm[384->1536,w_out_in,gelu_bwd]": 354.0e6,   # (forward with GELU, backward with GELU')
+    "esmm[384->1536,w_out_in,gelu_bwd+ess]": 354.0e6,   # (forward with GELU, backward with GELU' + bias-gradient sums)
 }
 
 

@@ -165,6 +165,47 @@ extern "C" int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y,
     return rc;
 }
 
+extern "C" int hexa_esmm_ess_ws_floats(int T, int k, int out_dim, int E, int64_t* out) {
+    if (!out || T < 0 || k < 1 || out_dim < 1 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm_ess_ws_floats: bad arguments");
+    // one row of column sums per (slot, 128-row tile, column tile); also enough for hexa_ess's 8 parts
+    const int64_t tiles = (int64_t)k * (T / HEXA_TILE_ROWS + E);
+    const int64_t cols = ((int64_t)out_dim + 255) / 256 * 256;
+    const int64_t a = tiles * cols, b = (int64_t)8 * E * out_dim;
+    *out = a > b ? a : b;
+    return HEXA_OK;
+}
+
+extern "C" int hexa_esmm_gelu_bwd_ess(void* out, void* db, const void* x, const void* w, const void* y1,
+                                      const int32_t* route, int w_layout, int db_accumulate, int T, int k, int in_dim,
+                                      int out_dim, int E, int x_dt, int w_dt, int db_dt, float* ws, int64_t ws_floats,
+                                      void* stream) {
+    if (int rc = check_sizes("hexa_esmm_gelu_bwd_ess", T, k, E, in_dim, out_dim)) return rc;
+    if (!out || !db || !x || !w || !y1 || !route) HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm_gelu_bwd_ess: null pointer");
+    if (!is_dt(x_dt) || !is_dt(w_dt) || !is_dt(db_dt)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm_gelu_bwd_ess: unknown element type");
+    int64_t need = 0;
+    hexa_esmm_ess_ws_floats(T, k, out_dim, E, &need);
+    if (T > 0 && is_16(x_dt) && w_dt == x_dt && ws && ws_floats >= need && dma_path_enabled()) {
+        EsmmArgs a;
+        a.out = out; a.x = x; a.w = w; a.bias = nullptr; a.out_act = const_cast<void*>(y1); a.slot_ws = nullptr;
+        a.r = route_view(route, T, k, E);
+        a.in_dim = in_dim; a.out_dim = out_dim;
+        a.x_per_slot = 0; a.out_per_slot = 1;
+        a.w_layout = w_layout; a.accumulate = 0;
+        a.x_dt = x_dt; a.w_dt = w_dt; a.bias_dt = HEXA_F32; a.out_dt = x_dt; a.act = HEXA_ACT_GELU_BWD;
+        if (w_layout != HEXA_W_IN_OUT && w_layout != HEXA_W_OUT_IN)
+            HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm_gelu_bwd_ess: bad w_layout %d", w_layout);
+        if (esmm16_dma_colsum_supported(a)) {
+            a.colsum = ws; a.db = db; a.db_dt = db_dt; a.db_accumulate = db_accumulate ? 1 : 0;
+            return launch_esmm16_dma(a, (hipStream_t)stream);
+        }
+    }
+    // any other case: the two operators one after the other (same results up to the order of the sums)
+    int rc = hexa_esmm(out, x, w, nullptr, route, 0, w_layout, 0, T, k, in_dim, out_dim, E, x_dt, w_dt, HEXA_F32, x_dt,
+                       HEXA_ACT_GELU_BWD, const_cast<void*>(y1), nullptr, stream);
+    if (rc) return rc;
+    return hexa_ess(db, out, route, 1, db_accumulate, T, k, out_dim, E, x_dt, db_dt, ws, ws ? ws_floats : 0, stream);
+}
+
 extern "C" int hexa_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, void* stream) {
     if (n < 0 || (n > 0 && (!dy1 || !dy2 || !y1))) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gelu_bwd: bad arguments");
     if (!is_dt(dt)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gelu_bwd: unknown element type");

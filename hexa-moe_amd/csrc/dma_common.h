@@ -264,6 +264,7 @@ struct EsmmK {
     int stream_out;   // results are stored with the streaming (non-temporal) hint
     long total;
     void* ws;   // slots > 0 write here ([slot-1][T][N]) when set: the slots are summed afterwards
+    float* colsum;   // when set: [slot][row tile][column tile][BN] column sums of the stored 16-bit result
 };
 
 inline int round_up(long v, int m) { return (int)(((v + m - 1) / m) * m); }

@@ -163,6 +163,11 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
     static_assert(PR * CP <= C::STAGE_AREA, "the staged result must fit in the stage buffers");
     constexpr int NPASS = OUT32 ? 1 : BM / PR;
     constexpr int RW = 32 * C::RB, FW = 32 * C::FB;
+    // column sums of the stored result (the bias gradient of the layer below): a thread of the store loop
+    // always handles the same 16-byte piece of a row when the workgroup size is a multiple of the pieces per row
+    constexpr bool COLSUM_OK = !OUT32 && C::NT % (BN / 8) == 0 && 64 % (BN / 8) == 0;
+    const bool colsum = COLSUM_OK && p.colsum != nullptr;
+    float cs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
         if (!OUT32) { if (pass == 0) barrier_nofence(); else __syncthreads(); }   // staging area is free
@@ -247,6 +252,14 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
                         val = make_uint4(vw[0], vw[1], vw[2], vw[3]);
                     }
                     store16(dst, val, p.stream_out == 1);
+                    if (colsum) {
+                        const unsigned vw[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            cs[2 * q] += from_bits16<TC>(vw[q] & 0xffff);
+                            cs[2 * q + 1] += from_bits16<TC>(vw[q] >> 16);
+                        }
+                    }
                     if (gelu) {
                         // applied to the value as stored (rounded), like act(y1) on the tensor
                         unsigned vw[4] = {val.x, val.y, val.z, val.w};
@@ -261,6 +274,52 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
             }
         }
     }
+    if (COLSUM_OK && colsum) {
+        constexpr int LPR = BN / 8;
+        // the 64 / LPR lanes of a wavefront that hold the same piece, then the wavefronts in order through LDS
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+#pragma unroll
+            for (int m = 32; m >= LPR; m >>= 1) cs[q] += __shfl_xor(cs[q], m);
+        }
+        __syncthreads();                          // the staged tile has been stored
+        float* red = reinterpret_cast<float*>(smem);
+        if (lane < LPR) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) red[wave * BN + lane * 8 + q] = cs[q];
+        }
+        __syncthreads();
+        float* dst = p.colsum + (((size_t)s * p.mt_ub + mt) * p.ntn + nt) * BN;
+        for (int c = tid; c < BN; c += C::NT) {
+            float t = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) t += red[w * BN + c];
+            dst[c] = t;
+        }
+    }
+}
+
+// db[e][n] (+)= the column sums of expert e's row tiles, slot after slot, tile after tile (fixed order).
+// Tile records are sorted by expert, so an expert's tiles of a slot are a contiguous run found by bisection.
+__global__ __launch_bounds__(256) void esmm_colsum_fold_kernel(void* __restrict__ db, const float* __restrict__ colsum,
+                                                               const int4* __restrict__ tile_info,
+                                                               const int32_t* __restrict__ tile_count, int mt_ub,
+                                                               int ntn, int bn, int N, int nslots, int db_dt,
+                                                               int accumulate) {
+    const int e = blockIdx.y;
+    const int n = blockIdx.x * 256 + threadIdx.x;
+    if (n >= N) return;
+    const int nt = n / bn, nl = n - nt * bn;
+    float sum = 0.f;
+    for (int s = 0; s < nslots; ++s) {
+        const int4* info = tile_info + (size_t)s * mt_ub;
+        const int cnt = min(tile_count[s], mt_ub);
+        int lo = 0, hi = cnt;          // first tile of an expert >= e
+        while (lo < hi) { const int mid = (lo + hi) >> 1; if (info[mid].x < e) lo = mid + 1; else hi = mid; }
+        for (int mt = lo; mt < cnt && info[mt].x == e; ++mt)
+            sum += colsum[(((size_t)s * mt_ub + mt) * ntn + nt) * bn + nl];
+    }
+    store_out(db, (size_t)e * N + n, sum, db_dt, accumulate != 0);
 }
 
 template <typename TC, bool IO, bool OUT32, typename C>
@@ -660,6 +719,7 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
     p.out_slot_rows = a.out_per_slot ? a.r.T : 0;
     p.bias_dt = a.bias_dt; p.out_dt = a.out_dt; p.act = a.act;
     p.stream_out = option(OPT_ESMM_STREAM) == 1;
+    p.colsum = a.colsum;
     p.group = p.ntn * (option(OPT_ESMM_GROUP) > 0 ? option(OPT_ESMM_GROUP) : (large ? 2 : 4));
     // Summing the slots into one result: with scratch, every slot runs in ONE launch (slot 0 into
     // `out`, the others into the scratch) and a reduction adds them in slot order; without it, one
@@ -685,6 +745,11 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
         if (rc) return rc;
     }
     if (p.ws) return launch_sum_slots(a.out, a.slot_ws, (int64_t)a.r.T * a.out_dim, a.r.k - 1, a.out_dt, st);
+    if (a.colsum) {
+        hipLaunchKernelGGL(esmm_colsum_fold_kernel, dim3(div_up(a.out_dim, 256), a.r.E), dim3(256), 0, st, a.db, a.colsum,
+                           p.tile_info, p.tile_count, p.mt_ub, p.ntn, C::BN, a.out_dim, a.r.k, a.db_dt, a.db_accumulate);
+        HEXA_CHECK_LAUNCH("esmm_colsum_fold");
+    }
     return HEXA_OK;
 }
 
@@ -743,6 +808,13 @@ int launch_estmm16_dma(const EstmmArgs& a, hipStream_t st) {
 // HEXA_MOE_PERSIST=1 selects the persistent-workgroup ESMM kernels (read once).  They are parity-
 // tested but not the default: on the shapes measured so far the one-tile-per-workgroup kernels win.
 static bool persist_enabled() { return option(OPT_PERSIST) == 1; }
+
+// The column sums ride on the store loop of the per-slot, 16-bit-result kernels (not the persistent one, not
+// the 128x384 tile, whose rows have 48 pieces).
+bool esmm16_dma_colsum_supported(const EsmmArgs& a) {
+    return esmm16_dma_supported(a) && a.out_dt == a.x_dt && a.out_per_slot && forced_tile() != 7 &&
+           !(persist_enabled() && esmm16_persist_supported(a));
+}
 
 int launch_esmm16_dma(const EsmmArgs& a, hipStream_t st) {
     if (persist_enabled() && esmm16_persist_supported(a)) return launch_esmm16_persist(a, forced_tile(), st);

@@ -56,6 +56,9 @@ struct EsmmArgs {
     int accumulate;                // result += instead of =
     int x_dt, w_dt, bias_dt, out_dt;
     int act;
+    // optional: also db[e][:] (+)= column sums of the expert's stored result rows (ESS of the result), through
+    // per-tile partial sums in `colsum` (16-bit per-slot results on the fast path only)
+    float* colsum = nullptr; void* db = nullptr; int db_dt = 0, db_accumulate = 0;
 };
 struct EstmmArgs {
     void* dw; const void* p; const void* q;   // dw[e][m][n] = sum_rows p[row][m] * q[row][n]
@@ -91,6 +94,7 @@ enum Opt {
 int option(int id);
 
 bool esmm16_dma_supported(const EsmmArgs& a);
+bool esmm16_dma_colsum_supported(const EsmmArgs& a);
 bool esmm16_persist_supported(const EsmmArgs& a);
 int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, hipStream_t st);
 int launch_esmm16_persist(const EsmmArgs& a, int tile, hipStream_t st);

@@ -41,6 +41,8 @@ SIGNATURES = {
     "hexa_ess": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
     "hexa_fused_grad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "hexa_gelu_bwd": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),
+    "hexa_esmm_ess_ws_floats": (_i, [_i, _i, _i, _i, ctypes.POINTER(_i64)]),
+    "hexa_esmm_gelu_bwd_ess": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
     "hexa_gate_logits": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "hexa_gate_ws_floats": (_i, [_i, _i, _i, ctypes.POINTER(_i64)]),
     "hexa_gate_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),

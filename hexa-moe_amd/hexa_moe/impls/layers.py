@@ -142,13 +142,19 @@ class FusedMoE_Shared_CudaCore(torch.autograd.Function):
             # [E, h, d_out]: the per-slot operand act(y1) supplies the rows of dW2
             dw2 = ops.estmm(y2, dy, route, True, False, out_dtype=grad_dtype(dt_w2)).to(dt_w2)
         if need_x or need_w1 or (ctx.has_b1 and need_b1):
-            if ctx.fused:   # dy1 = (dy . W2^T) * gelu'(y1) in the ESMM epilogue
+            bias1_done = False
+            if ctx.fused and ctx.has_b1 and need_b1:
+                # dy1 = (dy . W2^T) * gelu'(y1) and db1 = its per-expert row sums, from the same kernel
+                dy1, db1 = ops.esmm_gelu_bwd_ess(dy, w2, route, _lib.HEXA_W_OUT_IN, y1, db_dtype=grad_dtype(dt_b1))
+                db1 = db1.to(dt_b1)
+                bias1_done = True
+            elif ctx.fused:   # dy1 = (dy . W2^T) * gelu'(y1) in the ESMM epilogue
                 dy1 = ops.esmm(dy, w2, None, route, False, _lib.HEXA_W_OUT_IN, gelu_bwd_of=y1)
             else:
                 dy2 = ops.esmm(dy, w2, None, route, False, _lib.HEXA_W_OUT_IN)
                 (dy1,) = torch.autograd.grad(y2_graph, y1_leaf, dy2.to(y2_graph.dtype))
                 dy1 = dy1.to(x.dtype).contiguous()
-            if ctx.has_b1 and need_b1:
+            if ctx.has_b1 and need_b1 and not bias1_done:
                 db1 = ops.ess(dy1, route, True, out_dtype=grad_dtype(dt_b1)).to(dt_b1)
             if need_w1:
                 dw1 = ops.estmm(dy1, x, route, True, False, out_dtype=grad_dtype(dt_w1)).to(dt_w1)

@@ -270,6 +270,29 @@ def ess(dy, route, dy_per_slot, out=None, out_dtype=torch.float32, accumulate=Fa
     return out
 
 
+def esmm_gelu_bwd_ess(x, w, route, w_layout, y1, db_dtype=torch.float32):
+    """dy1 [k,T,out] = (x . w[e]) * gelu'(y1) and db [E,out] = per-expert row sums of dy1, in one call (the
+    sums ride on the producing kernel's store loop on the 16-bit fast path)."""
+    import ctypes
+    _dev(x, w, y1)
+    x, w, y1 = x.contiguous(), w.contiguous(), y1.contiguous()
+    T, k, E = route.T, route.k, route.E
+    in_dim = x.shape[-1]
+    out_dim = w.shape[2] if w_layout == _lib.HEXA_W_IN_OUT else w.shape[1]
+    assert tuple(x.shape) == (T, in_dim) and tuple(y1.shape) == (k, T, out_dim) and y1.dtype == x.dtype
+    out = torch.empty(k, T, out_dim, dtype=x.dtype, device=x.device)
+    db = torch.empty(E, out_dim, dtype=db_dtype, device=x.device)
+    n = ctypes.c_int64()
+    _lib.check(_lib.load().hexa_esmm_ess_ws_floats(T, k, out_dim, E, ctypes.byref(n)), "hexa_esmm_ess_ws_floats")
+    ws = torch.empty(int(n.value), dtype=torch.float32, device=x.device)
+    lay = "w_in_out" if w_layout == _lib.HEXA_W_IN_OUT else "w_out_in"
+    rc = _call(f"esmm[{in_dim}->{out_dim},{lay},gelu_bwd+ess]", _lib.load().hexa_esmm_gelu_bwd_ess, _ptr(out), _ptr(db),
+               _ptr(x), _ptr(w), _ptr(y1), _ptr(route.blob), int(w_layout), 0, T, k, in_dim, out_dim, E, _dt(x), _dt(w),
+               _dt(db), _ptr(ws), int(ws.numel()), _stream())
+    _lib.check(rc, "hexa_esmm_gelu_bwd_ess")
+    return out, db
+
+
 def gelu_bwd(dy2, y1):
     """dy1 = dy2 * gelu'(y1) (erf form)."""
     _dev(dy2, y1)

@@ -181,6 +181,18 @@ int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y, const void
                     int out_dim, int num_experts, int act_dt, int w_dt, int jx_dt, int jw_dt, int jb_dt,
                     void* slot_ws, void* stream);
 
+/* Steps 6-8 of the backward in one call: out[s][t][:] = (x[t][:] . w[e_s(t)]) * gelu'(y1[s][t][:]) (out, y1
+ * [k,T,out_dim] in x's type; no bias) and db[e][:] (+)= the sum of expert e's rows of `out` (ESS of the result).
+ * On the 16-bit fast path the column sums are taken in the producing kernel's store loop, per row tile, and
+ * folded in a fixed order, so `out` is not read again; otherwise hexa_esmm and hexa_ess run one after the other.
+ * ws: hexa_esmm_ess_ws_floats() floats (NULL: always the two-operator form).
+ * Replaces the ESMM task of FUSED_GRAD + activation jacobian + the ESS task of the next FUSED_GRAD
+ * (impls/layers.py:404-436, kernels/fused_ops_full.cu:372-431) for GELU. */
+int hexa_esmm_ess_ws_floats(int num_tokens, int top_k, int out_dim, int num_experts, int64_t* out);
+int hexa_esmm_gelu_bwd_ess(void* out, void* db, const void* x, const void* w, const void* y1, const int32_t* route,
+                           int w_layout, int db_accumulate, int num_tokens, int top_k, int in_dim, int out_dim,
+                           int num_experts, int x_dt, int w_dt, int db_dt, float* ws, int64_t ws_floats, void* stream);
+
 /* Elementwise backward of the fused GELU: dy1 = dy2 * gelu'(y1), n elements of type dt.  The
  * reference evaluates act' with torch.autograd.functional.jacobian (impls/layers.py:281-283,427). */
 int hexa_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, void* stream);

@@ -220,6 +220,38 @@ def test_esmm_fused_gelu_bwd(dev, dtype, d_in, d_out):
         assert_close(got, want, TOL[dtype], "esmm * gelu'")
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16, F16])
+@pytest.mark.parametrize("T,d_in,d_out,E,k,skew", [(1100, 96, 200, 5, 2, "zipf"), (2300, 384, 1536, 8, 2, None),
+                                                   (700, 64, 136, 4, 1, "one"), (37, 8, 8, 3, 1, None)])
+def test_esmm_gelu_bwd_with_bias_gradient(dev, dtype, T, d_in, d_out, E, k, skew):
+    """dy1 = (x . W[e]) * gelu'(y1) and db = per-expert row sums of dy1 from one call; the sums must be those
+    of the tensor as stored (what ESS of dy1 gives), and both must match the oracle."""
+    from hexa_moe import _lib, ops
+    print(f"esmm+gelu'+ess {dtype} T={T} in={d_in} out={d_out} E={E} k={k} {skew}", flush=True)
+    g = gen(T + d_out)
+    routing = make_routing(T, E, k, seed=T + 3, skew=skew, empty=1 if skew == "zipf" else 0)
+    _, offsets, token_ids = O.route_build(routing, E)
+    x = torch.randn(T, d_in, generator=g).to(dtype)
+    W = ((torch.rand(E, d_out, d_in, generator=g) * 2 - 1) / d_in ** 0.5).to(dtype)     # [E,out,in]
+    y1 = torch.randn(k, T, d_out, generator=g).to(dtype)
+    rd = _ref_dtype(dtype)
+    pre = O.esmm(x.to(rd), W.transpose(1, 2).to(rd), None, token_ids, offsets, False)
+    t = y1.to(rd)
+    want = pre * (0.5 * (1 + torch.erf(t / 2 ** 0.5)) + t * torch.exp(-0.5 * t * t) / (2 * torch.pi) ** 0.5)
+    route = ops.route_build(routing.to(dev), E)
+    got, db = ops.esmm_gelu_bwd_ess(x.to(dev), W.to(dev), route, _lib.HEXA_W_OUT_IN, y1.to(dev))
+    torch.cuda.synchronize()
+    tol = TOL[dtype]
+    assert got.dtype == dtype and db.dtype == F32 and db.shape == (E, d_out)
+    assert_close(got, want, tol, "dy1")
+    assert_close(db, O.ess(want, token_ids, offsets, True, E), tol, "db vs oracle")
+    # against the sums of the stored tensor: only the order of the fp32 additions differs
+    assert_close(db, O.ess(got.cpu().to(torch.float64), token_ids, offsets, True, E), 1e-5, "db vs stored dy1")
+    empty = (route.counts.sum(0) == 0).cpu()
+    if empty.any():
+        assert float(db.cpu()[empty].abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("pad", [1, 16])
 def test_reference_style_ops(dev, pad):
     """The five operator names of the reference extension, called the way impls/layers.py calls them:

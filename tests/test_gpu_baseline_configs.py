@@ -142,3 +142,28 @@ def test_skewed_stress_T32768_E64(dev):
     db2 = ops.ess(dyd * 2, route, True)
     torch.cuda.synchronize()
     assert torch.equal(dw2, dw * 2) and torch.equal(db2, db * 2)
+
+
+def test_large_token_count(dev):
+    """300 000 tokens (more than 2^16 units of every kind: rows, tiles, routing units), small dimensions:
+    every operator against the full oracle."""
+    from hexa_moe import _lib, ops
+    T, d_in, d_out, E, k = 300_000, 64, 72, 8, 2
+    print(f"config large T={T} in={d_in} out={d_out} E={E} k={k} bf16 seed=1239", flush=True)
+    g = gen(1239)
+    routing = make_routing(T, E, k, seed=1239)
+    x = torch.randn(T, d_in, generator=g).to(BF16)
+    W = uniform((E, d_in, d_out), 1 / math.sqrt(d_in), g).to(BF16)
+    b = uniform((E, d_out), 1 / math.sqrt(d_in), g).to(BF16)
+    dy = torch.randn(k, T, d_out, generator=g).to(BF16)
+    route = ops.route_build(routing.to(dev), E)
+    counts, offsets, token_ids = _check_route(route, routing, E)
+    tol = TOL[BF16]
+    y = ops.esmm(x.to(dev), W.to(dev), b.to(dev), route, False, _lib.HEXA_W_IN_OUT)
+    assert_close(y, O.esmm(x.float(), W.float(), b.float(), token_ids, offsets, False), tol, "esmm")
+    ys = ops.esmm(dy.to(dev), W.transpose(1, 2).contiguous().to(dev), None, route, True, _lib.HEXA_W_IN_OUT)
+    assert_close(ys, O.esmm(dy.float(), W.transpose(1, 2).float(), None, token_ids, offsets, True), tol, "esmm summed")
+    dw = ops.estmm(dy.to(dev), x.to(dev), route, True, False)
+    assert_close(dw, O.estmm(dy.float(), x.float(), token_ids, offsets, True, E), tol, "estmm")
+    db = ops.ess(dy.to(dev), route, True)
+    assert_close(db, O.ess(dy.float(), token_ids, offsets, True, E), tol, "ess")

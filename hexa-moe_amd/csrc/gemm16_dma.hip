@@ -800,8 +800,13 @@ int launch_estmm16_dma(const EstmmArgs& a, hipStream_t st) {
         case 8: return launch_estmm_dma_c<CfgS2>(a, st);
         case 9: return launch_estmm_dma_c<CfgS3>(a, st);
         case 1: return launch_estmm_dma_c<CfgS>(a, st);
-        // balanced units (a plan) keep 4 workgroups per CU busy; without a plan, more LDS per workgroup wins
-        default: return a.plan ? launch_estmm_dma_c<CfgS2>(a, st) : launch_estmm_dma_c<CfgS>(a, st);
+        // Balanced units (a plan) or short token lists keep 4 workgroups per CU busy (measured at 72 rows per
+        // expert, 3072 x 768: 105 -> 77 us); long lists without a plan are bounded by the busiest expert's
+        // walk, where deeper staging per workgroup wins.
+        default: {
+            const long avg_rows = (long)a.r.T * a.r.k / std::max(1, a.r.E);
+            return (a.plan || avg_rows < 512) ? launch_estmm_dma_c<CfgS2>(a, st) : launch_estmm_dma_c<CfgS>(a, st);
+        }
     }
 }
 

@@ -300,24 +300,44 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
 }
 
 // db[e][n] (+)= the column sums of expert e's row tiles, slot after slot, tile after tile (fixed order).
-// Tile records are sorted by expert, so an expert's tiles of a slot are a contiguous run found by bisection.
+// The tiles of a slot are listed expert after expert, so expert e's run starts at the number of tiles of the
+// experts before it: every thread of the workgroup adds up ceil(rows / tile_rows) over a share of those experts
+// (one round of loads instead of a bisection's chain of dependent ones).
 __global__ __launch_bounds__(256) void esmm_colsum_fold_kernel(void* __restrict__ db, const float* __restrict__ colsum,
-                                                               const int4* __restrict__ tile_info,
-                                                               const int32_t* __restrict__ tile_count, int mt_ub,
-                                                               int ntn, int bn, int N, int nslots, int db_dt,
-                                                               int accumulate) {
-    const int e = blockIdx.y;
-    const int n = blockIdx.x * 256 + threadIdx.x;
+                                                               const int32_t* __restrict__ offsets, int E, int mt_ub,
+                                                               int tile_rows, int ntn, int bn, int N, int nslots,
+                                                               int db_dt, int accumulate) {
+    __shared__ int sFirst[8], sCount[8];        // per slot: first tile of expert e, its number of tiles
+    __shared__ int red[256];
+    const int e = blockIdx.y, tid = threadIdx.x;
+    for (int s = 0; s < nslots; ++s) {
+        const int32_t* off = offsets + (size_t)s * (E + 1);
+        int before = 0;
+        for (int x = tid; x < e; x += 256) before += (off[x + 1] - off[x] + tile_rows - 1) / tile_rows;
+        red[tid] = before;
+        __syncthreads();
+        for (int w = 128; w > 0; w >>= 1) {
+            if (tid < w) red[tid] += red[tid + w];
+            __syncthreads();
+        }
+        if (tid == 0) { sFirst[s] = red[0]; sCount[s] = (off[e + 1] - off[e] + tile_rows - 1) / tile_rows; }
+        __syncthreads();
+    }
+    const int n = blockIdx.x * 256 + tid;
     if (n >= N) return;
     const int nt = n / bn, nl = n - nt * bn;
     float sum = 0.f;
     for (int s = 0; s < nslots; ++s) {
-        const int4* info = tile_info + (size_t)s * mt_ub;
-        const int cnt = min(tile_count[s], mt_ub);
-        int lo = 0, hi = cnt;          // first tile of an expert >= e
-        while (lo < hi) { const int mid = (lo + hi) >> 1; if (info[mid].x < e) lo = mid + 1; else hi = mid; }
-        for (int mt = lo; mt < cnt && info[mt].x == e; ++mt)
-            sum += colsum[(((size_t)s * mt_ub + mt) * ntn + nt) * bn + nl];
+        const int first = sFirst[s], last = min(first + sCount[s], mt_ub);
+        // eight loads in flight per trip (a busy expert has a dozen tiles; one load per trip would pay the
+        // memory latency a dozen times); the additions stay in tile order
+        for (int mt = first; mt < last; mt += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = colsum[(((size_t)s * mt_ub + min(mt + u, last - 1)) * ntn + nt) * bn + nl];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) sum += (mt + u < last) ? v[u] : 0.f;
+        }
     }
     store_out(db, (size_t)e * N + n, sum, db_dt, accumulate != 0);
 }
@@ -747,7 +767,8 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
     if (p.ws) return launch_sum_slots(a.out, a.slot_ws, (int64_t)a.r.T * a.out_dim, a.r.k - 1, a.out_dt, st);
     if (a.colsum) {
         hipLaunchKernelGGL(esmm_colsum_fold_kernel, dim3(div_up(a.out_dim, 256), a.r.E), dim3(256), 0, st, a.db, a.colsum,
-                           p.tile_info, p.tile_count, p.mt_ub, p.ntn, C::BN, a.out_dim, a.r.k, a.db_dt, a.db_accumulate);
+                           a.r.offsets, a.r.E, p.mt_ub, large ? HEXA_TILE_ROWS_L : HEXA_TILE_ROWS, p.ntn, C::BN, a.out_dim,
+                           a.r.k, a.db_dt, a.db_accumulate);
         HEXA_CHECK_LAUNCH("esmm_colsum_fold");
     }
     return HEXA_OK;
@@ -817,7 +838,7 @@ static bool persist_enabled() { return option(OPT_PERSIST) == 1; }
 // The column sums ride on the store loop of the per-slot, 16-bit-result kernels (not the persistent one, not
 // the 128x384 tile, whose rows have 48 pieces).
 bool esmm16_dma_colsum_supported(const EsmmArgs& a) {
-    return esmm16_dma_supported(a) && a.out_dt == a.x_dt && a.out_per_slot && forced_tile() != 7 &&
+    return esmm16_dma_supported(a) && a.out_dt == a.x_dt && a.out_per_slot && a.r.k <= 8 && forced_tile() != 7 &&
            !(persist_enabled() && esmm16_persist_supported(a));
 }
 

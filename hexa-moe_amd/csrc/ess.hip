@@ -106,8 +106,13 @@ __global__ __launch_bounds__(256) void ess_fold_kernel(void* __restrict__ db, co
                                                        int splits, int db_dt, int accumulate) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
-    float v = ws[i];
-    for (int z = 1; z < splits; ++z) v += ws[(size_t)z * n + i];
+    // all parts' loads in flight at once (at most 8 parts), added in part order
+    float part[8];
+#pragma unroll
+    for (int z = 0; z < 8; ++z) part[z] = ws[(size_t)min(z, splits - 1) * n + i];
+    float v = part[0];
+#pragma unroll
+    for (int z = 1; z < 8; ++z) v += z < splits ? part[z] : 0.f;
     store_out(db, (size_t)i, v, db_dt, accumulate != 0);
 }
 

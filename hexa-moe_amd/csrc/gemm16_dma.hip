@@ -434,10 +434,14 @@ __global__ __launch_bounds__(256) void estmm_fixup_kernel(void* __restrict__ dw,
     if (i >= mn) return;
     const int e = plan[r];
     const float* src = scratch + (size_t)plan[3 * E + r] * mn + i;
-    float4 v = *reinterpret_cast<const float4*>(src);
-    for (int c = 1; c < n; ++c) {
-        const float4 w = *reinterpret_cast<const float4*>(src + (size_t)c * mn);
-        v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+    // every part's load in flight at once (at most PLAN_MAX_PARTS), added in part order
+    float4 w[PLAN_MAX_PARTS];
+#pragma unroll
+    for (int c = 0; c < PLAN_MAX_PARTS; ++c) w[c] = *reinterpret_cast<const float4*>(src + (size_t)min(c, n - 1) * mn);
+    float4 v = w[0];
+#pragma unroll
+    for (int c = 1; c < PLAN_MAX_PARTS; ++c) {
+        if (c < n) { v.x += w[c].x; v.y += w[c].y; v.z += w[c].z; v.w += w[c].w; }
     }
     const size_t o = (size_t)e * mn + i;
     store_out(dw, o, v.x, dw_dt, accumulate != 0);

@@ -180,8 +180,20 @@ __global__ __launch_bounds__(256) void router_loss_kernel(float* __restrict__ l_
         const int c = i / E, e = i - c * E;
         const int b0 = c * per, b1 = min(nblocks, b0 + per);
         float m = 0.f, n = 0.f;
-#pragma unroll 4
-        for (int b = b0; b < b1; ++b) { m += part_me[(size_t)b * E + e]; n += part_cnt[(size_t)b * E + e]; }
+        for (int b = b0; b < b1; b += 8) {     // eight partials of each kind in flight per trip, added in order
+            float pm[8], pc[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const size_t at = (size_t)min(b + u, b1 - 1) * E + e;
+                pm[u] = part_me[at];
+                pc[u] = part_cnt[at];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                m += (b + u < b1) ? pm[u] : 0.f;
+                n += (b + u < b1) ? pc[u] : 0.f;
+            }
+        }
         s_m[i] = m;
         s_c[i] = n;
     }

@@ -29,6 +29,7 @@ SHAPES = [
     (1500, 264, 392, 16, 2, "zipf"),
     (1100, 512, 384, 8, 2, None),     # a 384-wide result: one tile spans it
     (900, 96, 328, 5, 2, "zipf"),
+    (500, 64, 72, 16, 8, None),       # eight slots: the most the fast path's slot tables hold
 ]
 
 

@@ -30,6 +30,7 @@ SHAPES = [
     (1100, 512, 384, 8, 2, None),     # a 384-wide result: one tile spans it
     (900, 96, 328, 5, 2, "zipf"),
     (500, 64, 72, 16, 8, None),       # eight slots: the most the fast path's slot tables hold
+    (300, 32, 40, 12, 9, None),       # nine: the general kernels take over where the tables end
 ]
 
 

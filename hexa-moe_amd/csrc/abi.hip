@@ -147,6 +147,20 @@ extern "C" int hexa_ess(void* db, const void* dy, const int32_t* route, int dy_p
     return launch_ess(a, st);
 }
 
+extern "C" int hexa_ess_noalloc(void* db, const void* dy, const int32_t* route, int dy_per_slot, int accumulate, int T,
+                                int k, int out_dim, int E, int dt, int db_dt, void* stream) {
+    if (int rc = check_sizes("hexa_ess_noalloc", T, k, E, out_dim, out_dim)) return rc;
+    if (!db || !route || !dy) HEXA_FAIL(HEXA_ERR_ARG, "hexa_ess_noalloc: null pointer");
+    if (!is_dt(dt) || !is_dt(db_dt)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_ess_noalloc: unknown element type");
+    EssArgs a;
+    a.db = db; a.dy = dy;
+    a.r = route_view(route, T, k, E);
+    a.out_dim = out_dim; a.dy_per_slot = dy_per_slot ? 1 : 0; a.accumulate = accumulate ? 1 : 0;
+    a.dy_dt = dt; a.db_dt = db_dt;
+    a.ws = nullptr; a.ws_floats = 0;
+    return launch_ess_noalloc(a, (hipStream_t)stream);
+}
+
 extern "C" int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y, const void* w, const void* x,
                                const int32_t* route, int m2s, int accumulate, int T, int k, int in_dim, int out_dim,
                                int E, int act_dt, int w_dt, int jx_dt, int jw_dt, int jb_dt, void* slot_ws,

@@ -237,6 +237,44 @@ int launch_ess(const EssArgs& a, hipStream_t st) {
     return launch_ess_t<_Float16>(a, st);
 }
 
+// ---- ESS without any allocation by anyone ---------------------------------------------------------------
+// The partial sums of the split walk live in a file-scope device array instead of caller scratch.  Every
+// device the library runs on holds its own copy at its own address; the array's name is only a host-side
+// handle, so the device address is looked up once per device (with that device current) and kept.
+constexpr int64_t ESS_SCRATCH_FLOATS = HEXA_ESS_NOALLOC_MAX_FLOATS;   // 8 MiB per device
+constexpr int ESS_MAX_DEVICES = 64;
+static __device__ __align__(256) float scratch[ESS_SCRATCH_FLOATS];
+static float* g_scratch_ptr[ESS_MAX_DEVICES];
+
+int ess_scratch_for_current_device(float** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= ESS_MAX_DEVICES)
+        HEXA_FAIL(HEXA_ERR_LAUNCH, "hexa_ess_noalloc: cannot identify the current device");
+    if (!g_scratch_ptr[dev]) {
+        float* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            HEXA_FAIL(HEXA_ERR_LAUNCH, "hexa_ess_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return HEXA_OK;
+}
+
+int launch_ess_noalloc(EssArgs a, hipStream_t st) {
+    const int64_t need = (int64_t)8 * a.r.E * a.out_dim;
+    if (need > ESS_SCRATCH_FLOATS)
+        HEXA_FAIL(HEXA_ERR_UNSUPPORTED,
+                  "hexa_ess_noalloc: 8*num_experts*out_dim = %lld floats exceeds the built-in scratch of %lld floats; "
+                  "use hexa_ess with caller scratch", (long long)need, (long long)ESS_SCRATCH_FLOATS);
+    float* ptr = nullptr;
+    if (int rc = ess_scratch_for_current_device(&ptr)) return rc;
+    // every partial sum the fold reads is written by this call's own workgroups: nothing to clear
+    a.ws = ptr;
+    a.ws_floats = need;
+    return launch_ess(a, st);
+}
+
 int launch_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, hipStream_t st) {
     if (dt == HEXA_F32) return launch_gelu_bwd_t<float>(dy1, dy2, y1, n, st);
     if (dt == HEXA_BF16) return launch_gelu_bwd_t<__bf16>(dy1, dy2, y1, n, st);

@@ -105,6 +105,7 @@ int launch_estmm16_dma(const EstmmArgs& a, hipStream_t s);
 int launch_estmm16(const EstmmArgs& a, hipStream_t s);
 int launch_estmm32(const EstmmArgs& a, hipStream_t s);
 int launch_ess(const EssArgs& a, hipStream_t s);
+int launch_ess_noalloc(EssArgs a, hipStream_t s);
 int launch_sum_slots(void* out, const void* ws, int64_t n, int nws, int dt, hipStream_t s);
 int launch_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, hipStream_t s);
 

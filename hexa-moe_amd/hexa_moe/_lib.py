@@ -39,6 +39,7 @@ SIGNATURES = {
     "hexa_estmm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp]),
     "hexa_estmm_plan": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
     "hexa_ess": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
+    "hexa_ess_noalloc": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "hexa_fused_grad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "hexa_gelu_bwd": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),
     "hexa_esmm_ess_ws_floats": (_i, [_i, _i, _i, _i, ctypes.POINTER(_i64)]),

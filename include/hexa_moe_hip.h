@@ -166,6 +166,19 @@ int hexa_estmm_plan(int32_t* plan, const int32_t* route, int num_tokens, int top
 int hexa_ess(void* db, const void* dy, const int32_t* route, int dy_per_slot, int accumulate, int num_tokens,
              int top_k, int out_dim, int num_experts, int dt, int db_dt, float* ws, int64_t ws_floats, void* stream);
 
+/* hexa_ess for callers that cannot allocate or hand over scratch (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the same kernels and the same split walk as hexa_ess with
+ * 8*num_experts*out_dim floats of scratch, so the results are bit-identical to that call, but the partial sums
+ * live in an array built into the library (HEXA_ESS_NOALLOC_MAX_FLOATS floats per device, held until the
+ * process ends).  8*num_experts*out_dim beyond that limit is rejected with HEXA_ERR_UNSUPPORTED.  The call
+ * allocates and frees nothing.  All calls on one device share the array: calls that overlap on one GPU (two
+ * streams, two threads) race; calls on one stream are ordered and safe.  The device of `stream` must be the
+ * current device.  No counterpart in the reference (its ESS task allocates nothing because it walks each
+ * list in one thread block, kernels/fused_ops_full.cu:372-431). */
+#define HEXA_ESS_NOALLOC_MAX_FLOATS (2 * 1024 * 1024)
+int hexa_ess_noalloc(void* db, const void* dy, const int32_t* route, int dy_per_slot, int accumulate,
+                     int num_tokens, int top_k, int out_dim, int num_experts, int dt, int db_dt, void* stream);
+
 /* The reference's fused backward of one expert linear:
  *   j_x[(s),t,:in] (+)= j_y[(s),t,:out] . w[e]      w [E][out][in]
  *   j_w[e]         (+)= sum j_y^T x                 j_w [E][out][in]

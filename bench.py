@@ -28,15 +28,24 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
 T, D, H, E, K_TOP = 18432, 384, 1536, 32, 2
 SEED = 1235
 
-# HBM bytes per launch (fetch + write) of the matmul kernels on this workload, from rocprofv3 FETCH_SIZE /
-# WRITE_SIZE counter passes scaled by a plain elementwise kernel of known size (--calibrate-copy); the
-# commands and the per-kernel figures are in profiles/*.hbm_traffic.txt.  Keys are the per-op labels.
-MEASURED_TRAFFIC_BYTES = {
-    "estmm[1536x384]": 408.8e6 + 40.1e6,            # main kernel + the fixup of the experts cut into parts
-    "esmm[1536->384,w_in_out,sum_slots]": 234.4e6 + 42.5e6,   # + the slot sum
-    "esmm[384->1536,w_out_in,gelu]": 354.0e6,       # average over the two launches of this kernel
-    "esmm[384->1536,w_out_in,gelu_bwd+ess]": 354.0e6,   # (forward with GELU, backward with GELU' + bias-gradient sums)
-}
+# The six matmul launches of a step, in the order the library's event pairs number them: (direction, pair index).
+MAJOR = [("fc1_esmm+gelu", "fwd", 0), ("fc2_esmm+slot_sum", "fwd", 1), ("dy1_esmm+gelu'+colsum", "bwd", 0),
+         ("dx_esmm+slot_sum", "bwd", 1), ("dW2_estmm", "bwd", 2), ("dW1_estmm", "bwd", 3)]
+ROOFLINE_KERNEL = "fc1_esmm+gelu"   # fixed: the launch with the largest share of the step among equal-FLOP matmuls
+
+
+def measured_traffic(label):
+    """HBM bytes per launch (fetch + write) of a matmul launch, read from the `@traffic <label> <fetch_bytes>
+    <write_bytes>` lines of profiles/*.hbm_traffic.txt (rocprofv3 FETCH_SIZE / WRITE_SIZE passes scaled by a
+    copy kernel of known size; the commands are in that file).  None when no profile covers the label."""
+    import glob
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.hbm_traffic.txt"))):
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 4 and parts[0] == "@traffic" and parts[1] == label:
+                    return float(parts[2]) + float(parts[3])
+    return None
 
 
 def make_module_and_inputs(dev):
@@ -88,7 +97,7 @@ def main():
     import torch
     import torch.nn.functional as F
 
-    from hexa_moe import _lib, ops
+    from hexa_moe import _lib
 
     _lib.load()  # no fallback: a missing library is an error
     dev = torch.device("cuda:0")
@@ -102,7 +111,7 @@ def main():
             prm.grad = None
         y, l_aux = m(0, x)
         torch.autograd.backward([y, l_aux], [dy, one])
-        return y, m.dispatch_params.indices_
+        return y, m.dispatch_params.routing_
 
     if args.calibrate_copy:   # known traffic: 2^27 bf16 read + 2^27 bf16 written per launch
         src = torch.ones(1 << 27, dtype=torch.bfloat16, device=dev)
@@ -112,83 +121,66 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # Warm-up.  Its last steps carry an event pair around EVERY operator call (the per-operator table of the
-    # output); the timed steps carry events only around the calls of the operator that dominates the step,
-    # so that `value` is not inflated by ~50 event records per step (measured: 0.82 ms with them, 0.72 without).
-    survey_steps = 0 if args.no_kernel_events else min(args.warmup, 5)
-    for _ in range(args.warmup - survey_steps):
+    from hexa_moe.impls.layers import FusedMoEDepth
+
+    for _ in range(args.warmup):
         step()
-    survey = None
-    if survey_steps:
-        survey = ops.OpTimer()
-        ops.set_timer(survey)
-        for _ in range(survey_steps):
-            step()
-        ops.set_timer(None)
-    dom_label = f"estmm[{H}x{D}]"
-    if survey is not None:
-        tot = {label: sum(v) for label, v in survey.durations().items()}
-        dom_label = max(tot, key=tot.get)
-    timer = None if args.no_kernel_events else ops.OpTimer(only=[dom_label])
-    ops.set_timer(timer)
+    # Event pairs around the six matmul launches are recorded by the library itself on the launch stream
+    # (hexa_moe_depth_forward / _backward take caller-owned events).  One pair per timed step, in rotation: a
+    # record costs a few microseconds of stream time, and one per step keeps `value` honest.
+    pairs = []
+    if not args.no_kernel_events:
+        for _ in range(args.steps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(); b.record()           # creates the handles
+            pairs.append((a, b))
     torch.cuda.synchronize()
+    host = 0.0
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for i in range(args.steps):
+        if pairs:
+            _, direction, j = MAJOR[i % len(MAJOR)]
+            arr = [None] * 8
+            arr[2 * j], arr[2 * j + 1] = pairs[i]
+            FusedMoEDepth.events = {"fwd": arr if direction == "fwd" else None, "bwd": arr if direction == "bwd" else None}
         y, idx = step()
+    host = time.perf_counter() - t0            # the host has enqueued every step; the device is still running
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    ops.set_timer(None)
+    FusedMoEDepth.events = None
     ms = (t1 - t0) * 1e3 / args.steps
+    host_us = host * 1e6 / args.steps
     flops_step = 12.0 * T * K_TOP * D * H
     tokens_per_s = T / (ms * 1e-3)
 
-    # ---- per-operator durations (events on the launch stream) ----
+    # ---- the six matmul launches, timed inside the timed steps ----
     kernels = {}
     roofline = None
-    if timer is not None:
+    if pairs:
         gemm = 2.0 * T * K_TOP * D * H
-        esz = 2  # bf16
-        alg = {  # algorithmic work per call: flop for the matmuls, bytes for the HBM-bound kernels
-            "route_build": ("hbm", T * K_TOP * 4 + T * K_TOP * 8 + K_TOP * (2 * E + 1) * 4),
-            "gate_logits": ("hbm", T * D * esz + E * D * 4 + T * E * 4),
-            "router_forward": ("hbm", 2 * T * E * 4 + T * K_TOP * 4),
-            "router_backward": ("hbm", 2 * T * E * 4),
-            "estmm_plan": ("hbm", K_TOP * (E + 1) * 4 + (4 * E + 1) * 4),
-            "gate_backward": ("hbm", T * D * esz * 2 + T * E * 4 + 2 * E * D * 4),
-            "gelu_bwd": ("hbm", 3 * T * K_TOP * H * esz),
-            f"ess[{H},per_slot]": ("hbm", T * K_TOP * H * esz + E * H * esz),
-            f"ess[{D}]": ("hbm", T * K_TOP * D * esz + E * D * esz),
-        }
-        per_op = {label: (vals, survey_steps) for label, vals in (survey.durations().items() if survey else [])}
-        per_op.update({label: (vals, args.steps) for label, vals in timer.durations().items()})   # timed region wins
-        for label, (vals, nsteps) in per_op.items():
+        samples = {}
+        for i, (a, b) in enumerate(pairs):
+            samples.setdefault(MAJOR[i % len(MAJOR)][0], []).append(a.elapsed_time(b))   # ms
+        for label, vals in samples.items():
             avg_ms = statistics.mean(vals)
-            per_step = len(vals) / nsteps
-            kind, work = alg.get(label, ("mfma", gemm))
-            entry = {"avg_us": round(avg_ms * 1e3, 2), "calls_per_step": per_step, "bound": kind}
-            if kind == "mfma":
-                entry["tflops"] = round(work / (avg_ms * 1e-3) / 1e12, 1)
-                entry["frac"] = round(entry["tflops"] / PEAK_BF16_TFLOPS, 4)
-            else:
-                entry["gbs"] = round(work / (avg_ms * 1e-3) / 1e9, 1)
-                entry["frac"] = round(entry["gbs"] / PEAK_HBM_GBS, 4)
-            kernels[label] = entry
-        dom = dom_label
-        d = kernels[dom]
-        d["measured_in"] = "timed steps"
-        if d["bound"] == "mfma":
-            roofline = {"kernel": dom, "bound": "mfma", "achieved": d["tflops"], "peak": PEAK_BF16_TFLOPS,
-                        "unit": "TFLOP/s", "frac": d["frac"], "traffic": MEASURED_TRAFFIC_BYTES.get(dom)}
-        else:
-            roofline = {"kernel": dom, "bound": "hbm", "achieved": d["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                        "frac": d["frac"], "traffic": None}
+            tf = gemm / (avg_ms * 1e-3) / 1e12
+            kernels[label] = {"avg_us": round(avg_ms * 1e3, 2), "samples": len(vals), "bound": "mfma",
+                              "tflops": round(tf, 1), "frac": round(tf / PEAK_BF16_TFLOPS, 4)}
+        if ROOFLINE_KERNEL in kernels:
+            d = kernels[ROOFLINE_KERNEL]
+            roofline = {"kernel": ROOFLINE_KERNEL, "bound": "mfma", "achieved": d["tflops"], "peak": PEAK_BF16_TFLOPS,
+                        "unit": "TFLOP/s", "frac": d["frac"], "traffic": measured_traffic(ROOFLINE_KERNEL),
+                        "algorithmic_flop": gemm, "avg_us": d["avg_us"]}
 
     # ---- CPU baseline: the oracle's plain-PyTorch fp32 evaluation of the same layer on the host ----
     cpu = None
     parity = None
     if not args.no_cpu_baseline:
         from oracle import hexa_oracle as O
-        threads = min(16, os.cpu_count() or 1)
+        # as many threads as the box grants this process: its CPU share (OMP_NUM_THREADS, 16 per GPU on the
+        # benchmark boxes) or, where none is set, every logical CPU
+        logical = os.cpu_count() or 1
+        threads = max(1, min(logical, int(os.environ.get("OMP_NUM_THREADS", logical))))
         torch.set_num_threads(threads)
         c = {"x": x, "W1": m.batched_fc1_w[0], "W2": m.batched_fc2_w[0], "b1": m.batched_fc1_bias[0],
              "b2": m.batched_fc2_bias[0], "dy": dy}
@@ -202,10 +194,11 @@ def main():
             ref = run()
             times.append(time.perf_counter() - a)
         sec = statistics.median(times)
-        cpu = {"value": round(T / sec, 1), "unit": "tokens/s", "cores": threads, "kind": "port",
+        cpu = {"value": round(T / sec, 1), "unit": "tokens/s", "cores": threads, "threads": threads,
+               "host_logical_cpus": logical, "kind": "port",
                "gflops": round(flops_step / sec / 1e9, 1),
                "sample": f"the full workload (T={T}, one layer fwd+bwd, fp32, per-expert index_select/mm/index_add), "
-                         f"1 warm-up + median of 3 on {threads} threads"}
+                         f"1 warm-up + median of 3 on {threads} threads of {logical} logical CPUs"}
         names = ["y", "dx", "dW1", "dW2", "db1", "db2"]
         got = [y, x.grad, m.batched_fc1_w[0].grad, m.batched_fc2_w[0].grad, m.batched_fc1_bias[0].grad,
                m.batched_fc2_bias[0].grad]
@@ -224,9 +217,10 @@ def main():
                    "routing": "top-2 of softmax(x.wg), logits ~ N(0,1) + N(0,0.5) per-expert bias"},
         "tflops": round(flops_step / (ms * 1e-3) / 1e12, 1),
         "frac_bf16_mfma_peak": round(flops_step / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+        "host_enqueue_us_per_step": round(host_us, 1),
         "roofline": roofline, "cpu_baseline": cpu, "parity_rel_err_vs_cpu": parity, "kernels": kernels,
-        "kernels_note": "HIP events on the launch stream; the roofline kernel's calls are timed inside the timed steps, "
-                        "the other operators in the last warm-up steps",
+        "kernels_note": "the six matmul launches, each timed by a HIP event pair the library records on the launch stream, "
+                        "one launch per timed step in rotation; every other kernel of the step is in profiles/*.kernel_stats.txt",
     }
     print(json.dumps(out))
 

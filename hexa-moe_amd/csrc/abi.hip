@@ -66,10 +66,13 @@ extern "C" int hexa_set_option(const char* name, int value) {
 extern "C" const char* hexa_last_error(void) { return g_err; }
 extern "C" int hexa_abi_version(void) { return HEXA_ABI_VERSION; }
 
-extern "C" int hexa_esmm(void* out, const void* x, const void* w, const void* bias, const int32_t* route, int m2s,
-                         int w_layout, int accumulate, int T, int k, int in_dim, int out_dim, int E, int x_dt,
-                         int w_dt, int bias_dt, int out_dt, int act, void* out_act, void* slot_ws,
-                         void* stream) {
+// The body of hexa_esmm with one more operand: `sum_extra` (may be null) is a tensor of the result's shape that
+// the slot sum adds on the fast path (m2s, top_k > 1, slot_ws given); *extra_used says whether it was added.
+int hexa::esmm_call(void* out, const void* x, const void* w, const void* bias, const int32_t* route, int m2s,
+                    int w_layout, int accumulate, int T, int k, int in_dim, int out_dim, int E, int x_dt, int w_dt,
+                    int bias_dt, int out_dt, int act, void* out_act, void* slot_ws, const void* sum_extra,
+                    bool* extra_used, void* stream) {
+    if (extra_used) *extra_used = false;
     if (int rc = check_sizes("hexa_esmm", T, k, E, in_dim, out_dim)) return rc;
     if (!out || !x || !w || !route) HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: null pointer");
     if (w_layout != HEXA_W_IN_OUT && w_layout != HEXA_W_OUT_IN) HEXA_FAIL(HEXA_ERR_ARG, "hexa_esmm: bad w_layout %d", w_layout);
@@ -100,8 +103,22 @@ extern "C" int hexa_esmm(void* out, const void* x, const void* w, const void* bi
         HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_esmm: result must be fp32 or the tokens' 16-bit type");
     if (bias && bias_dt != x_dt && bias_dt != HEXA_F32)
         HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_esmm: bias must be fp32 or the tokens' 16-bit type");
-    if (dma_path_enabled() && esmm16_dma_supported(a)) return launch_esmm16_dma(a, st);
+    if (dma_path_enabled() && esmm16_dma_supported(a)) {
+        if (sum_extra && !a.out_per_slot && k > 1 && slot_ws) {
+            a.sum_extra = sum_extra;
+            if (extra_used) *extra_used = true;
+        }
+        return launch_esmm16_dma(a, st);
+    }
     return launch_esmm16(a, st);
+}
+
+extern "C" int hexa_esmm(void* out, const void* x, const void* w, const void* bias, const int32_t* route, int m2s,
+                         int w_layout, int accumulate, int T, int k, int in_dim, int out_dim, int E, int x_dt,
+                         int w_dt, int bias_dt, int out_dt, int act, void* out_act, void* slot_ws,
+                         void* stream) {
+    return esmm_call(out, x, w, bias, route, m2s, w_layout, accumulate, T, k, in_dim, out_dim, E, x_dt, w_dt, bias_dt,
+                     out_dt, act, out_act, slot_ws, nullptr, nullptr, stream);
 }
 
 extern "C" int hexa_estmm(void* dw, const void* dy, const void* x, const int32_t* route, int dy_per_slot,

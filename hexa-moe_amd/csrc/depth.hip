@@ -1,0 +1,241 @@
+// One MoE depth per call: hexa_moe_depth_forward / hexa_moe_depth_backward enqueue every kernel of a depth
+// (gate projection, softmax + top-k + auxiliary loss, routing segment pass, the ten steps of the formula table
+// with the exact GELU) through the single-operator entry points of this library, in the order the Python layer
+// used to call them.  Nothing here allocates: all scratch is carved out of one caller-owned workspace.
+//
+// Replaces the MoE branch of MoE_Cascaded.forward (hexa_moe_cuda/hexa_moe/impls/cascaded_moe.py:508-568),
+// FusedMoE_Shared_CudaCore.forward (impls/layers.py:99-277) and .backward (impls/layers.py:280-474).
+#include <algorithm>
+
+#include "hexa_internal.h"
+
+namespace hexa {
+namespace {
+
+constexpr int64_t WS_ALIGN = 256;
+
+int64_t elem_size(int dt) { return dt == HEXA_F32 ? 4 : 2; }
+bool known_dt(int dt) { return dt == HEXA_F32 || dt == HEXA_F16 || dt == HEXA_BF16; }
+
+struct Carver {   // hands out aligned pieces of the workspace; with base == nullptr it only measures
+    char* base; int64_t used = 0;
+    explicit Carver(void* b) : base(static_cast<char*>(b)) {}
+    void* take(int64_t bytes) {
+        void* p = base ? base + used : nullptr;
+        used += (bytes + WS_ALIGN - 1) / WS_ALIGN * WS_ALIGN;
+        return p;
+    }
+};
+
+// ESTMM scratch slots for the busiest experts' partial results (the same rule as the Python wrapper of the
+// single operator: up to 2E slots, at most 256 MiB, only for 16-bit operands with long enough lists)
+int estmm_slots(const hexa_moe_depth_desc& d, int out_dim, int in_dim) {
+    if (d.act_dt == HEXA_F32 || (int64_t)d.num_tokens * d.top_k < (int64_t)128 * d.num_experts) return 0;
+    const int64_t mn = (int64_t)out_dim * in_dim;
+    if (mn % 4) return 0;
+    const int64_t slots = std::min<int64_t>(2 * d.num_experts, ((int64_t)256 << 20) / (mn * 4));
+    return slots >= 2 ? (int)slots : 0;
+}
+
+struct FwdWs { float* router; void* slot_ws; int64_t bytes; };
+struct BwdWs {
+    float* dlogits; float* gate; float* ess; float* colsum; int64_t colsum_floats; int32_t* plan; float* estmm;
+    int slots; void* slot_ws; void* dx_gate; int64_t bytes;
+};
+
+int carve_forward(const hexa_moe_depth_desc& d, void* ws, FwdWs* out) {
+    Carver c(ws);
+    int64_t rf = 0;
+    if (int rc = hexa_router_ws_floats(d.num_tokens, d.num_experts, &rf)) return rc;
+    out->router = static_cast<float*>(c.take(rf * 4));
+    out->slot_ws = d.top_k > 1 ? c.take((int64_t)(d.top_k - 1) * d.num_tokens * d.d_out * elem_size(d.act_dt)) : nullptr;
+    out->bytes = c.used;
+    return HEXA_OK;
+}
+
+int carve_backward(const hexa_moe_depth_desc& d, void* ws, BwdWs* out) {
+    Carver c(ws);
+    const int T = d.num_tokens, k = d.top_k, E = d.num_experts;
+    int64_t gf = 0, cf = 0;
+    if (int rc = hexa_gate_ws_floats(T, d.d_in, E, &gf)) return rc;
+    if (int rc = hexa_esmm_ess_ws_floats(T, k, d.hidden, E, &cf)) return rc;
+    out->dlogits = static_cast<float*>(c.take((int64_t)T * E * 4));
+    out->gate = static_cast<float*>(c.take(gf * 4));
+    out->ess = static_cast<float*>(c.take((int64_t)8 * E * d.d_out * 4));
+    out->colsum = static_cast<float*>(c.take(cf * 4));
+    out->colsum_floats = cf;
+    // one plan and one scratch area serve both ESTMM calls (they run one after the other on the stream)
+    const int s2 = estmm_slots(d, d.hidden, d.d_out), s1 = estmm_slots(d, d.hidden, d.d_in);
+    out->slots = std::min(s1, s2);
+    out->plan = static_cast<int32_t*>(c.take((int64_t)(4 * E + 1) * 4));
+    out->estmm = out->slots >= 2
+                     ? static_cast<float*>(c.take((int64_t)out->slots * d.hidden * std::max(d.d_in, d.d_out) * 4))
+                     : nullptr;
+    out->slot_ws = k > 1 ? c.take((int64_t)(k - 1) * T * d.d_in * elem_size(d.act_dt)) : nullptr;
+    out->dx_gate = c.take((int64_t)T * d.d_in * elem_size(d.act_dt));
+    out->bytes = c.used;
+    return HEXA_OK;
+}
+
+int check_desc(const char* who, const hexa_moe_depth_desc* d) {
+    if (!d) HEXA_FAIL(HEXA_ERR_ARG, "%s: null descriptor", who);
+    if (d->num_tokens < 1 || d->top_k < 1 || d->num_experts < 1 || d->d_in < 1 || d->hidden < 1 || d->d_out < 1)
+        HEXA_FAIL(HEXA_ERR_ARG, "%s: bad sizes T=%d k=%d E=%d dims=(%d,%d,%d)", who, d->num_tokens, d->top_k,
+                  d->num_experts, d->d_in, d->hidden, d->d_out);
+    if (d->top_k > d->num_experts) HEXA_FAIL(HEXA_ERR_ARG, "%s: top_k exceeds the number of experts", who);
+    if (!known_dt(d->act_dt) || !known_dt(d->w_dt)) HEXA_FAIL(HEXA_ERR_ARG, "%s: unknown element type", who);
+    if (d->loss != 0 && d->loss != 1) HEXA_FAIL(HEXA_ERR_ARG, "%s: loss must be 0 (GShard) or 1 (load-importance)", who);
+    return HEXA_OK;
+}
+
+struct EventPairs {   // caller-owned events recorded around the major kernels (null handles are skipped)
+    void* const* ev; int n; hipStream_t st;
+    int begin(int i) const {
+        if (ev && 2 * i + 1 < n && ev[2 * i] && hipEventRecord((hipEvent_t)ev[2 * i], st) != hipSuccess)
+            HEXA_FAIL(HEXA_ERR_LAUNCH, "hipEventRecord failed");
+        return HEXA_OK;
+    }
+    int end(int i) const {
+        if (ev && 2 * i + 1 < n && ev[2 * i + 1] && hipEventRecord((hipEvent_t)ev[2 * i + 1], st) != hipSuccess)
+            HEXA_FAIL(HEXA_ERR_LAUNCH, "hipEventRecord failed");
+        return HEXA_OK;
+    }
+};
+
+}  // namespace
+}  // namespace hexa
+
+using namespace hexa;
+
+#define RUN(call)                 \
+    do {                          \
+        if (int rc__ = (call)) return rc__; \
+    } while (0)
+
+extern "C" int hexa_moe_depth_ws_bytes(const hexa_moe_depth_desc* d, int64_t* forward_bytes, int64_t* backward_bytes) {
+    RUN(check_desc("hexa_moe_depth_ws_bytes", d));
+    if (forward_bytes) {
+        FwdWs f;
+        RUN(carve_forward(*d, nullptr, &f));
+        *forward_bytes = std::max<int64_t>(f.bytes, WS_ALIGN);
+    }
+    if (backward_bytes) {
+        BwdWs b;
+        RUN(carve_backward(*d, nullptr, &b));
+        *backward_bytes = std::max<int64_t>(b.bytes, WS_ALIGN);
+    }
+    return HEXA_OK;
+}
+
+extern "C" int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* x, const float* wg, const float* noise,
+                                      const void* fc1_w, const void* fc1_b, const void* fc2_w, const void* fc2_b,
+                                      float* logits, float* scores, int32_t* idx, float* thr, float* stats,
+                                      int32_t* route, void* y1, void* y2, void* y, void* ws, int64_t ws_bytes,
+                                      void* const* events, int num_events, void* stream) {
+    const char* who = "hexa_moe_depth_forward";
+    RUN(check_desc(who, d));
+    if (!x || !fc1_w || !fc2_w || !idx || !route || !y1 || !y2 || !y || !ws) HEXA_FAIL(HEXA_ERR_ARG, "%s: null pointer", who);
+    if (((uintptr_t)ws & (WS_ALIGN - 1)) != 0) HEXA_FAIL(HEXA_ERR_ARG, "%s: the workspace must be 256-byte aligned", who);
+    FwdWs w;
+    RUN(carve_forward(*d, ws, &w));
+    if (ws_bytes < w.bytes) HEXA_FAIL(HEXA_ERR_ARG, "%s: workspace of %lld bytes, %lld needed", who, (long long)ws_bytes, (long long)w.bytes);
+    const int T = d->num_tokens, k = d->top_k, E = d->num_experts;
+    const EventPairs ev{events, num_events, (hipStream_t)stream};
+    if (wg) {
+        if (!logits || !scores || !stats || (d->loss == 1 && !thr)) HEXA_FAIL(HEXA_ERR_ARG, "%s: null router state", who);
+        RUN(hexa_gate_logits(logits, x, wg, T, d->d_in, E, d->act_dt, stream));
+        if (d->loss == 0)
+            RUN(hexa_router_forward(scores, idx, stats, stats + E, stats + 2 * E, logits, noise, d->noise_scale, T, E, k,
+                                    w.router, stream));
+        else
+            RUN(hexa_router_forward_load_importance(scores, idx, thr, stats, stats + E, stats + 2 * E, stats + 3 * E,
+                                                    stats + 4 * E, logits, noise, d->noise_scale, d->sigma, T, E, k,
+                                                    w.router, stream));
+    }
+    RUN(hexa_route_build(idx, 0, k, 1, T, k, E, route, stream));
+    RUN(ev.begin(0));
+    RUN(hexa_esmm(y1, x, fc1_w, fc1_b, route, 0, HEXA_W_OUT_IN, 0, T, k, d->d_in, d->hidden, E, d->act_dt, d->w_dt,
+                  d->b1_dt, d->act_dt, HEXA_ACT_GELU, y2, nullptr, stream));
+    RUN(ev.end(0));
+    RUN(ev.begin(1));
+    RUN(hexa_esmm(y, y2, fc2_w, fc2_b, route, 1, HEXA_W_IN_OUT, 0, T, k, d->hidden, d->d_out, E, d->act_dt, d->w_dt,
+                  d->b2_dt, d->act_dt, HEXA_ACT_NONE, nullptr, w.slot_ws, stream));
+    RUN(ev.end(1));
+    return HEXA_OK;
+}
+
+extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void* dy, const float* grad_l_aux,
+                                       const void* x, const float* wg, const void* fc1_w, const void* fc2_w,
+                                       const float* scores, const int32_t* idx, const float* thr, const float* stats,
+                                       const int32_t* route, const void* y1, const void* y2, void* dx, float* dwg,
+                                       void* dw1, void* db1, void* dw2, void* db2, void* dy1, void* ws,
+                                       int64_t ws_bytes, void* const* events, int num_events, void* stream) {
+    const char* who = "hexa_moe_depth_backward";
+    RUN(check_desc(who, d));
+    if (!dy || !x || !fc1_w || !fc2_w || !route || !y1 || !y2 || !dy1 || !ws) HEXA_FAIL(HEXA_ERR_ARG, "%s: null pointer", who);
+    if (((uintptr_t)ws & (WS_ALIGN - 1)) != 0) HEXA_FAIL(HEXA_ERR_ARG, "%s: the workspace must be 256-byte aligned", who);
+    BwdWs w;
+    RUN(carve_backward(*d, ws, &w));
+    if (ws_bytes < w.bytes) HEXA_FAIL(HEXA_ERR_ARG, "%s: workspace of %lld bytes, %lld needed", who, (long long)ws_bytes, (long long)w.bytes);
+    const int T = d->num_tokens, k = d->top_k, E = d->num_experts;
+    const EventPairs ev{events, num_events, (hipStream_t)stream};
+    const bool gate_path = wg && grad_l_aux && (dx || dwg);
+    if (gate_path && (!scores || !stats || (d->loss == 1 && (!thr || !idx)))) HEXA_FAIL(HEXA_ERR_ARG, "%s: null router state", who);
+
+    // step 4: db2 = ESS(dy)
+    if (db2) RUN(hexa_ess(db2, dy, route, 0, 0, T, k, d->d_out, E, d->act_dt, d->gb2_dt, w.ess, (int64_t)8 * E * d->d_out, stream));
+    const bool planned = w.slots >= 2 && (dw1 || dw2);
+    if (planned) RUN(hexa_estmm_plan(w.plan, route, T, k, E, w.slots, stream));
+    // step 5: dW2 = ESTMM(act(y1), dy): the per-slot operand supplies the rows of dW2 [E][hidden][d_out]
+    if (dw2) {
+        RUN(ev.begin(2));
+        RUN(hexa_estmm(dw2, y2, dy, route, 1, 0, 0, T, k, d->hidden, d->d_out, E, d->act_dt, d->gw2_dt,
+                       planned ? w.plan : nullptr, planned ? w.slots : 0, planned ? w.estmm : nullptr, stream));
+        RUN(ev.end(2));
+    }
+    if (dx || dw1 || db1) {
+        // steps 6-8: dy1 = (dy . W2^T) * gelu'(y1), db1 = ESS(dy1)
+        RUN(ev.begin(0));
+        if (db1)
+            RUN(hexa_esmm_gelu_bwd_ess(dy1, db1, dy, fc2_w, y1, route, HEXA_W_OUT_IN, 0, T, k, d->d_out, d->hidden, E,
+                                       d->act_dt, d->w_dt, d->gb1_dt, w.colsum, w.colsum_floats, stream));
+        else
+            RUN(hexa_esmm(dy1, dy, fc2_w, nullptr, route, 0, HEXA_W_OUT_IN, 0, T, k, d->d_out, d->hidden, E, d->act_dt,
+                          d->w_dt, HEXA_F32, d->act_dt, HEXA_ACT_GELU_BWD, const_cast<void*>(y1), nullptr, stream));
+        RUN(ev.end(0));
+        // step 9: dW1 = ESTMM(dy1, x)
+        if (dw1) {
+            RUN(ev.begin(3));
+            RUN(hexa_estmm(dw1, dy1, x, route, 1, 0, 0, T, k, d->hidden, d->d_in, E, d->act_dt, d->gw1_dt,
+                           planned ? w.plan : nullptr, planned ? w.slots : 0, planned ? w.estmm : nullptr, stream));
+            RUN(ev.end(3));
+        }
+    }
+    // the gate path: d l_aux / d logits through the softmax (and the threshold), then through the projection
+    bool gate_dx_in_ws = false;
+    if (gate_path) {
+        if (d->loss == 0)
+            RUN(hexa_router_backward(w.dlogits, scores, stats + E, grad_l_aux, T, E, stream));
+        else
+            RUN(hexa_router_backward_load_importance(w.dlogits, scores, thr, idx, stats + 2 * E, stats + 3 * E, grad_l_aux,
+                                                     d->sigma, T, E, k, stream));
+        // With several slots on the 16-bit fast path the slot sum of step 10 adds the gate's share as one more
+        // addend; otherwise the gate's share is written into dx first and step 10 accumulates onto it.
+        gate_dx_in_ws = dx && k > 1 && d->act_dt != HEXA_F32 && d->w_dt == d->act_dt && dma_path_enabled() &&
+                        (d->hidden % 32) == 0 && (d->d_in % 8) == 0;
+        RUN(hexa_gate_backward(dx ? (gate_dx_in_ws ? w.dx_gate : dx) : nullptr, dwg, w.dlogits, x, wg, T, d->d_in, E,
+                               d->act_dt, w.gate, stream));
+    }
+    // step 10: dx = ESMM(dy1, W1), summed over the slots (+ the gate's share)
+    if (dx) {
+        RUN(ev.begin(1));
+        bool used = false;
+        const int acc = gate_path && !gate_dx_in_ws ? 1 : 0;
+        RUN(esmm_call(dx, dy1, fc1_w, nullptr, route, 1, HEXA_W_IN_OUT, acc, T, k, d->hidden, d->d_in, E, d->act_dt,
+                      d->w_dt, HEXA_F32, d->act_dt, HEXA_ACT_NONE, nullptr, w.slot_ws, gate_dx_in_ws ? w.dx_gate : nullptr,
+                      &used, stream));
+        if (gate_dx_in_ws && !used) HEXA_FAIL(HEXA_ERR_LAUNCH, "%s: internal: the gate's input gradient was not added", who);
+        RUN(ev.end(1));
+    }
+    return HEXA_OK;
+}

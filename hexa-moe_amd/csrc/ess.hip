@@ -189,9 +189,10 @@ int launch_gelu_bwd_t(void* dy1, const void* dy2, const void* y1, int64_t n, hip
 
 // out[i] += ws[0][i] + ws[1][i] + ... in fp32, slot order (the deterministic reduction behind the
 // one-launch slot sum of ESMM)
+// `extra` (may be null): one more addend of out's shape, added last (the gate path's share of an input gradient)
 template <typename T>
 __global__ __launch_bounds__(256) void sum_slots_kernel(T* __restrict__ out, const T* __restrict__ ws, int64_t n,
-                                                        int nws) {
+                                                        int nws, const T* __restrict__ extra) {
     constexpr int V = Vec16<T>::N;
     const int64_t nv = n / V;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -206,6 +207,11 @@ __global__ __launch_bounds__(256) void sum_slots_kernel(T* __restrict__ out, con
 #pragma unroll
             for (int j = 0; j < V; ++j) acc[j] += Cvt<T>::to_f(w.e[j]);
         }
+        if (extra) {
+            w.u = reinterpret_cast<const uint4*>(extra)[i];
+#pragma unroll
+            for (int j = 0; j < V; ++j) acc[j] += Cvt<T>::to_f(w.e[j]);
+        }
 #pragma unroll
         for (int j = 0; j < V; ++j) o.e[j] = Cvt<T>::from_f(acc[j]);
         reinterpret_cast<uint4*>(out)[i] = o.u;
@@ -213,22 +219,23 @@ __global__ __launch_bounds__(256) void sum_slots_kernel(T* __restrict__ out, con
 }
 
 template <typename T>
-int launch_sum_slots_t(void* out, const void* ws, int64_t n, int nws, hipStream_t st) {
-    if (n == 0 || nws == 0) return HEXA_OK;
+int launch_sum_slots_t(void* out, const void* ws, int64_t n, int nws, const void* extra, hipStream_t st) {
+    if (n == 0 || (nws == 0 && !extra)) return HEXA_OK;
     if (n % Vec16<T>::N) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "sum_slots: size must be a multiple of the vector width");
     int64_t blocks = (n / Vec16<T>::N + 255) / 256;
     if (blocks > 256 * 16) blocks = 256 * 16;
-    hipLaunchKernelGGL((sum_slots_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, (T*)out, (const T*)ws, n, nws);
+    hipLaunchKernelGGL((sum_slots_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, (T*)out, (const T*)ws, n, nws,
+                       (const T*)extra);
     HEXA_CHECK_LAUNCH("sum_slots");
     return HEXA_OK;
 }
 
 }  // namespace
 
-int launch_sum_slots(void* out, const void* ws, int64_t n, int nws, int dt, hipStream_t st) {
-    if (dt == HEXA_F32) return launch_sum_slots_t<float>(out, ws, n, nws, st);
-    if (dt == HEXA_BF16) return launch_sum_slots_t<__bf16>(out, ws, n, nws, st);
-    return launch_sum_slots_t<_Float16>(out, ws, n, nws, st);
+int launch_sum_slots(void* out, const void* ws, int64_t n, int nws, int dt, hipStream_t st, const void* extra) {
+    if (dt == HEXA_F32) return launch_sum_slots_t<float>(out, ws, n, nws, extra, st);
+    if (dt == HEXA_BF16) return launch_sum_slots_t<__bf16>(out, ws, n, nws, extra, st);
+    return launch_sum_slots_t<_Float16>(out, ws, n, nws, extra, st);
 }
 
 int launch_ess(const EssArgs& a, hipStream_t st) {

@@ -768,7 +768,7 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
                                            : launch_esmm_dma_d<_Float16, C>(p, grid, io, o32, st);
         if (rc) return rc;
     }
-    if (p.ws) return launch_sum_slots(a.out, a.slot_ws, (int64_t)a.r.T * a.out_dim, a.r.k - 1, a.out_dt, st);
+    if (p.ws) return launch_sum_slots(a.out, a.slot_ws, (int64_t)a.r.T * a.out_dim, a.r.k - 1, a.out_dt, st, a.sum_extra);
     if (a.colsum) {
         hipLaunchKernelGGL(esmm_colsum_fold_kernel, dim3(div_up(a.out_dim, 256), a.r.E), dim3(256), 0, st, a.db, a.colsum,
                            a.r.offsets, a.r.E, p.mt_ub, large ? HEXA_TILE_ROWS_L : HEXA_TILE_ROWS, p.ntn, C::BN, a.out_dim,

@@ -694,7 +694,7 @@ int launch_c(const EsmmArgs& a, bool large, hipStream_t st) {
         const int rc = a.x_dt == HEXA_BF16 ? launch_d<__bf16, C>(p, io, o32, st) : launch_d<_Float16, C>(p, io, o32, st);
         if (rc) return rc;
     }
-    if (p.ws) return launch_sum_slots(a.out, a.slot_ws, (int64_t)a.r.T * a.out_dim, a.r.k - 1, a.out_dt, st);
+    if (p.ws) return launch_sum_slots(a.out, a.slot_ws, (int64_t)a.r.T * a.out_dim, a.r.k - 1, a.out_dt, st, a.sum_extra);
     return HEXA_OK;
 }
 

@@ -59,6 +59,8 @@ struct EsmmArgs {
     // optional: also db[e][:] (+)= column sums of the expert's stored result rows (ESS of the result), through
     // per-tile partial sums in `colsum` (16-bit per-slot results on the fast path only)
     float* colsum = nullptr; void* db = nullptr; int db_dt = 0, db_accumulate = 0;
+    // optional, with slot_ws on the fast path: one more tensor of the result's shape added by the slot sum
+    const void* sum_extra = nullptr;
 };
 struct EstmmArgs {
     void* dw; const void* p; const void* q;   // dw[e][m][n] = sum_rows p[row][m] * q[row][n]
@@ -76,6 +78,9 @@ struct EssArgs {
     float* ws; int64_t ws_floats;   // optional scratch for partial sums
 };
 
+int esmm_call(void* out, const void* x, const void* w, const void* bias, const int32_t* route, int m2s, int w_layout,
+              int accumulate, int T, int k, int in_dim, int out_dim, int E, int x_dt, int w_dt, int bias_dt, int out_dt,
+              int act, void* out_act, void* slot_ws, const void* sum_extra, bool* extra_used, void* stream);
 int launch_esmm16(const EsmmArgs& a, hipStream_t s);
 int launch_esmm32(const EsmmArgs& a, hipStream_t s);
 // Tuning / testing knobs: 0 = automatic.  Each one starts from an environment variable (read once) and
@@ -106,7 +111,7 @@ int launch_estmm16(const EstmmArgs& a, hipStream_t s);
 int launch_estmm32(const EstmmArgs& a, hipStream_t s);
 int launch_ess(const EssArgs& a, hipStream_t s);
 int launch_ess_noalloc(EssArgs a, hipStream_t s);
-int launch_sum_slots(void* out, const void* ws, int64_t n, int nws, int dt, hipStream_t s);
+int launch_sum_slots(void* out, const void* ws, int64_t n, int nws, int dt, hipStream_t s, const void* extra = nullptr);
 int launch_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, hipStream_t s);
 
 // ---- small device helpers -------------------------------------------------------------------

@@ -79,10 +79,13 @@ __global__ __launch_bounds__(ROUTER_TB) void router_fwd_kernel(float* __restrict
         }
     }
     __syncthreads();
+    // The selection is total: a row of NaN scores (NaN or +Inf logits) beats no entry, so the list starts out
+    // as experts 0..k-1 and such a token stays routed (torch.topk also returns valid ids for NaN rows); its
+    // NaN then reaches the output through the token's own features and the loss through the score sums.
     float best_v[MAX_TOPK];
     int best_i[MAX_TOPK];
 #pragma unroll
-    for (int j = 0; j < MAX_TOPK; ++j) { best_v[j] = -INFINITY; best_i[j] = 0x7fffffff; }
+    for (int j = 0; j < MAX_TOPK; ++j) { best_v[j] = -INFINITY; best_i[j] = j; }
     if (STAGED) {
         float* col = tile + lane;          // this token's values, ROUTER_P apart
         float mx = -INFINITY;
@@ -271,7 +274,7 @@ __global__ __launch_bounds__(ROUTER_TB) void router_li_fwd_kernel(float* __restr
     float best_v[MAX_TOPK];
     int best_i[MAX_TOPK];
 #pragma unroll
-    for (int j = 0; j < MAX_TOPK; ++j) { best_v[j] = -INFINITY; best_i[j] = 0x7fffffff; }
+    for (int j = 0; j < MAX_TOPK; ++j) { best_v[j] = -INFINITY; best_i[j] = j; }
     // noisy scores: selection only
     float mx = -INFINITY, cmx = -INFINITY;
     for (int e = 0; e < E; ++e) {

@@ -27,6 +27,13 @@ class RouteLayout(ctypes.Structure):
                 ("reserved", ctypes.c_int32)]
 
 
+class DepthDesc(ctypes.Structure):
+    """hexa_moe_depth_desc of include/hexa_moe_hip.h."""
+    _fields_ = [(n, ctypes.c_int32) for n in ("num_tokens", "top_k", "num_experts", "d_in", "hidden", "d_out", "act_dt",
+                                              "w_dt", "b1_dt", "b2_dt", "gw1_dt", "gw2_dt", "gb1_dt", "gb2_dt", "loss")] + \
+               [("noise_scale", ctypes.c_float), ("sigma", ctypes.c_float), ("reserved", ctypes.c_int32)]
+
+
 # name -> (restype, argtypes); kept in one table so the export test can walk it
 SIGNATURES = {
     "hexa_route_layout_get": (_i, [_i, _i, _i, ctypes.POINTER(RouteLayout)]),
@@ -53,6 +60,9 @@ SIGNATURES = {
     "hexa_router_forward_load_importance": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float,
                                                  ctypes.c_float, _i, _i, _i, _vp, _vp]),
     "hexa_router_backward_load_importance": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float, _i, _i, _i, _vp]),
+    "hexa_moe_depth_ws_bytes": (_i, [ctypes.POINTER(DepthDesc), ctypes.POINTER(_i64), ctypes.POINTER(_i64)]),
+    "hexa_moe_depth_forward": (_i, [ctypes.POINTER(DepthDesc)] + [_vp] * 16 + [_vp, _i64, _vp, _i, _vp]),
+    "hexa_moe_depth_backward": (_i, [ctypes.POINTER(DepthDesc)] + [_vp] * 20 + [_vp, _i64, _vp, _i, _vp]),
     "hexa_last_error": (ctypes.c_char_p, []),
     "hexa_abi_version": (_i, []),
     "hexa_set_option": (_i, [ctypes.c_char_p, _i]),
@@ -75,7 +85,7 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.hexa_abi_version() != 5:
+    if lib.hexa_abi_version() != 6:
         raise RuntimeError("hexa_moe: libhexa_moe_hip.so has an unexpected ABI version")
     _lib = lib
     return lib

@@ -34,7 +34,8 @@ from torch import nn
 
 from .. import ops
 from . import losses, router
-from .layers import FusedMoE_Shared_CudaCore, MLP_Implement, simplified_extract_critical, topk_and_loss  # noqa: F401
+from .layers import (FusedMoE_Shared_CudaCore, FusedMoEDepth, MLP_Implement, is_plain_gelu,  # noqa: F401
+                     simplified_extract_critical, topk_and_loss)
 
 
 def cast_if_autocast_enabled(tensor):
@@ -126,6 +127,7 @@ class MoE_Cascaded(nn.Module):
         self.use_2dh = use_2dh
         self.parallel_type = parallel_type
         self.fused_router = True   # set False to route with the PyTorch formulation
+        self.fused_depth = True    # set False to run a depth operator by operator instead of as two library calls
         # One device holds every expert in full; a process group, if there is one, only replicates.
         self.world_size, self.local_rank = 1, 0
         if dist.is_available() and dist.is_initialized():
@@ -178,7 +180,7 @@ class MoE_Cascaded(nn.Module):
             has_fc1_bias=mlp_fc1_bias, has_fc2_bias=mlp_fc2_bias, data_centric=True,
             input_dim_list_moe=self.input_dim_list_moe, output_dim_list_moe=self.output_dim_list_moe,
             hidden_size_list_moe=self.hidden_size_list_moe, local_dim_list=self.local_dim_list,
-            num_global_experts=E, indices_=None, route_pool=RoutePool())
+            num_global_experts=E, indices_=None, routing_=None, route_pool=RoutePool())
 
         self._init_moe()
         self._build_gates(gate_type, seeds)
@@ -283,6 +285,12 @@ class MoE_Cascaded(nn.Module):
                                                    self.num_global_experts, gate.gate_noise)
         return topk_and_loss(scores, top_k, loss_fn)
 
+    def _depth_call_supported(self, gate, x, top_k):
+        """The one-call-per-depth path covers the linear fp32 gate with the fused router and the exact GELU."""
+        return (self.fused_depth and self.fused_router and is_plain_gelu(self.dispatch_params.activation_fn)
+                and router.fused_route_supported(gate, x, top_k, self.num_global_experts, self.is_gshard_loss)
+                and (gate.fp32_gate or x.dtype == torch.float32))
+
     def forward(self, depth_idx, input, gate_index=0, top_k=None, a2a_ffn_overlap_degree=None, reserve_dims=1):
         is_moe = depth_idx in self.moe_idx_list
         if self.skip_moe:
@@ -309,12 +317,22 @@ class MoE_Cascaded(nn.Module):
         gate = self.gates[i * self.gate_len + gate_index]
         if a2a_ffn_overlap_degree is not None:
             self.a2a_ffn_overlap_degree = a2a_ffn_overlap_degree
-        indices, l_aux = self._route(gate, x, top_k or gate.top_k)
-
         cfg = self.dispatch_params
-        cfg.indices_ = indices  # [T,k] int64, read in place by the routing pass
         cfg.stage = i
-        y = FusedMoE_Shared_CudaCore.apply(cfg, x.contiguous(), self.batched_fc1_w[i], self.batched_fc2_w[i],
-                                           self.batched_fc1_bias[i], self.batched_fc2_bias[i]).to(original_dtype)
+        k = min(int(top_k or gate.top_k), self.num_global_experts)
+        if self._depth_call_supported(gate, x, k):
+            # the whole depth as two library calls (forward, backward)
+            noise_scale = gate.gate_noise / self.num_global_experts if (self.training and gate.gate_noise > 0) else 0.0
+            opts = (k, noise_scale, bool(self.is_gshard_loss), gate.gate_noise / self.num_global_experts)
+            y, l_aux = FusedMoEDepth.apply(cfg, opts, x.contiguous(), gate.wg.weight, self.batched_fc1_w[i],
+                                           self.batched_fc2_w[i], self.batched_fc1_bias[i], self.batched_fc2_bias[i])
+            y = y.to(original_dtype)
+        else:
+            indices, l_aux = self._route(gate, x, k)
+            cfg.routing_ = indices  # [T,k] int64 / int32, read in place by the routing pass
+            y = FusedMoE_Shared_CudaCore.apply(cfg, x.contiguous(), self.batched_fc1_w[i], self.batched_fc2_w[i],
+                                               self.batched_fc1_bias[i], self.batched_fc2_bias[i]).to(original_dtype)
+        # the reference's form of the decision (cascaded_moe.py:545): k int32 vectors of T expert ids
+        cfg.indices_ = [col.to(torch.int32) for col in cfg.routing_.unbind(dim=1)]
         y = y.view(list(original_shape[:-reserve_dims]) + list(y.shape[-reserve_dims:]))
         return (self.result_func(y) if self.result_func is not None else y), l_aux

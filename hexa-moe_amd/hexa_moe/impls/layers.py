@@ -84,7 +84,9 @@ class FusedMoE_Shared_CudaCore(torch.autograd.Function):
         assert fc1_w.shape[0] == E and fc2_w.shape[0] == E and fc1_w.shape[2] == d_in
         assert fc1_w.shape[1] == fc2_w.shape[1]
 
-        indices = config.indices_
+        indices = getattr(config, "routing_", None)   # [T,k] tensor; else the reference's list of k vectors
+        if indices is None:
+            indices = config.indices_
         routing = indices if torch.is_tensor(indices) else torch.stack([i.reshape(-1) for i in indices], dim=1)
         blob = config.route_pool.slot(config.stage, T, routing.shape[1], E, x.device)
         route = ops.route_build(routing, E, blob=blob)
@@ -163,6 +165,115 @@ class FusedMoE_Shared_CudaCore(torch.autograd.Function):
         ctx.act_graph = None
         ctx.config.stage = ctx.config.stage - 1
         return (None, dx, dw1, dw2, db1, db2)
+
+
+class _BlobOwner:
+    """Keeps a route-pool slot bound while a backward that reads it is pending."""
+
+    def __init__(self, blob):
+        self.blob = blob
+
+
+class FusedMoEDepth(torch.autograd.Function):
+    """One MoE depth -- gate projection, softmax + top-k + auxiliary loss, the routing segment pass and the
+    MoE FFN with the exact GELU -- as TWO library calls (hexa_moe_depth_forward / _backward) instead of one
+    call per operator: the same kernels in the same order as the linear gate's routing followed by
+    FusedMoE_Shared_CudaCore (reference: impls/cascaded_moe.py:508-568 and impls/layers.py:99-474), with the
+    gate path's share of dx added inside the expert path's slot sum.  Returns (y, l_aux)."""
+
+    events = None   # optional {"fwd": [torch.cuda.Event, ...], "bwd": [...]} recorded around the major kernels
+
+    @staticmethod
+    def forward(ctx: Any, config: Any, opts: Any, tokens_input, wg, fc1_w, fc2_w, fc1_bias, fc2_bias):
+        top_k, noise_scale, is_gshard, sigma = opts
+        x = tokens_input.contiguous()
+        E = int(config.num_global_experts)
+        T, d_in = x.shape
+        hidden, d_out = fc1_w.shape[1], fc2_w.shape[2]
+        assert fc1_w.shape == (E, hidden, d_in) and fc2_w.shape[:2] == (E, hidden) and wg.shape == (E, d_in)
+        w1, w2 = _weight_for(x, fc1_w, T * top_k), _weight_for(x, fc2_w, T * top_k)
+        if w1.dtype != w2.dtype:
+            w1, w2 = w1.to(x.dtype), w2.to(x.dtype)
+        w1, w2, wg32 = w1.contiguous(), w2.contiguous(), wg.float().contiguous()
+        b1 = fc1_bias.contiguous() if fc1_bias is not None else None
+        b2 = fc2_bias.contiguous() if fc2_bias is not None else None
+
+        def grad_dtype(p):   # fp32 master parameters get fp32 gradients, 16-bit parameters 16-bit ones
+            return None if p is None else (torch.float32 if p.dtype == torch.float32 else x.dtype)
+
+        key = (T, top_k, E, d_in, hidden, d_out, x.dtype, w1.dtype, None if b1 is None else b1.dtype,
+               None if b2 is None else b2.dtype, fc1_w.dtype, fc2_w.dtype, is_gshard, float(noise_scale), float(sigma))
+        plans = config.__dict__.setdefault("depth_plans", {})
+        plan = plans.get(key)
+        if plan is None:
+            plan = plans[key] = ops.DepthPlan(T, top_k, E, d_in, hidden, d_out, x.dtype, w1.dtype,
+                                              None if b1 is None else b1.dtype, None if b2 is None else b2.dtype,
+                                              grad_dtype(fc1_w), grad_dtype(fc2_w), grad_dtype(fc1_bias) or torch.float32,
+                                              grad_dtype(fc2_bias) or torch.float32, 0 if is_gshard else 1,
+                                              noise_scale, sigma)
+        dev = x.device
+        nstats = (2 if is_gshard else 4) * E + 1
+        state = torch.empty(2 * T * E + T + nstats, dtype=torch.float32, device=dev)
+        logits, scores = state[:T * E], state[T * E:2 * T * E]
+        thr, stats = state[2 * T * E:2 * T * E + T], state[2 * T * E + T:]
+        idx = torch.empty(T, top_k, dtype=torch.int32, device=dev)
+        noise = torch.randn(T, E, dtype=torch.float32, device=dev) if noise_scale > 0 else None
+        blob = config.route_pool.slot(config.stage, T, top_k, E, dev)
+        y12 = torch.empty(2, top_k, T, hidden, dtype=x.dtype, device=dev)
+        y = torch.empty(T, d_out, dtype=x.dtype, device=dev)
+        ws = torch.empty(plan.fwd_bytes, dtype=torch.uint8, device=dev)
+        ev = FusedMoEDepth.events
+        ops.moe_depth_forward(plan, x, wg32, noise, w1, b1, w2, b2, logits, scores, idx, None if is_gshard else thr, stats,
+                              blob, y12[0], y12[1], y, ws, ev["fwd"] if ev else None)
+        config.routing_ = idx
+        if any(ctx.needs_input_grad):
+            ctx.owner = _BlobOwner(blob)
+            config.route_pool.bind(config.stage, ctx.owner)   # keep the slot until this call's backward is done
+        ctx.config, ctx.plan, ctx.is_gshard = config, plan, is_gshard
+        ctx.param_dtypes = (wg.dtype, fc1_w.dtype, fc2_w.dtype, None if fc1_bias is None else fc1_bias.dtype,
+                            None if fc2_bias is None else fc2_bias.dtype)
+        ctx.dims = (T, top_k, E, d_in, hidden, d_out)
+        ctx.save_for_backward(x, wg32, w1, w2, state, idx, y12, blob)
+        ctx.set_materialize_grads(False)
+        return y, stats[nstats - 1]
+
+    @staticmethod
+    def backward(ctx: Any, dy, dl_aux):
+        x, wg32, w1, w2, state, idx, y12, blob = ctx.saved_tensors
+        T, top_k, E, d_in, hidden, d_out = ctx.dims
+        dev = x.device
+        need_x, need_wg, need_w1, need_w2, need_b1, need_b2 = ctx.needs_input_grad[2:8]
+        dt_wg, dt_w1, dt_w2, dt_b1, dt_b2 = ctx.param_dtypes
+        dy = torch.zeros(T, d_out, dtype=x.dtype, device=dev) if dy is None else dy.contiguous().to(x.dtype)
+        g_aux = None if dl_aux is None else dl_aux.to(torch.float32).contiguous()
+
+        def grad_dtype(p):
+            return torch.float32 if p == torch.float32 else x.dtype
+
+        def new(shape, dtype, want):
+            return torch.empty(shape, dtype=dtype, device=dev) if want else None
+
+        dx = new((T, d_in), x.dtype, need_x)
+        dwg = new((E, d_in), torch.float32, need_wg and g_aux is not None)
+        dw1 = new((E, hidden, d_in), grad_dtype(dt_w1), need_w1)
+        dw2 = new((E, hidden, d_out), grad_dtype(dt_w2), need_w2)
+        db1 = new((E, hidden), grad_dtype(dt_b1), dt_b1 is not None and need_b1)
+        db2 = new((E, d_out), grad_dtype(dt_b2), dt_b2 is not None and need_b2)
+        dy1 = torch.empty(top_k, T, hidden, dtype=x.dtype, device=dev)
+        ws = torch.empty(ctx.plan.bwd_bytes, dtype=torch.uint8, device=dev)
+        nstats = (2 if ctx.is_gshard else 4) * E + 1
+        scores = state[T * E:2 * T * E]
+        thr, stats = state[2 * T * E:2 * T * E + T], state[2 * T * E + T:2 * T * E + T + nstats]
+        ev = FusedMoEDepth.events
+        ops.moe_depth_backward(ctx.plan, dy, g_aux, x, wg32, w1, w2, scores, idx, None if ctx.is_gshard else thr, stats,
+                               blob, y12[0], y12[1], dx, dwg, dw1, db1, dw2, db2, dy1, ws, ev["bwd"] if ev else None)
+        ctx.owner = None
+        ctx.config.stage = ctx.config.stage - 1
+
+        def cast(g, dt):
+            return None if g is None else g.to(dt)
+
+        return (None, None, dx, cast(dwg, dt_wg), cast(dw1, dt_w1), cast(dw2, dt_w2), cast(db1, dt_b1), cast(db2, dt_b2))
 
 
 def topk_and_loss(scores, top_k, loss_fn=losses.gshard_loss):

@@ -416,3 +416,55 @@ def router_backward_load_importance(scores, thr, idx, stats, grad_l_aux, sigma):
                T, E, int(idx.shape[1]), _stream())
     _lib.check(rc, "hexa_router_backward_load_importance")
     return dlogits
+
+
+# ---- one MoE depth per call ---------------------------------------------------------------------------------
+class DepthPlan:
+    """Descriptor and workspace sizes of hexa_moe_depth_forward / _backward for one (shape, dtypes, loss)."""
+
+    def __init__(self, T, k, E, d_in, hidden, d_out, act_dtype, w_dtype, b1_dtype, b2_dtype, gw1, gw2, gb1, gb2,
+                 loss, noise_scale, sigma):
+        import ctypes
+        dt = lambda t: _DT[t] if t is not None else 0   # noqa: E731
+        self.desc = _lib.DepthDesc(int(T), int(k), int(E), int(d_in), int(hidden), int(d_out), dt(act_dtype), dt(w_dtype),
+                                   dt(b1_dtype), dt(b2_dtype), dt(gw1), dt(gw2), dt(gb1), dt(gb2), int(loss),
+                                   float(noise_scale), float(sigma), 0)
+        f, b = ctypes.c_int64(), ctypes.c_int64()
+        _lib.check(_lib.load().hexa_moe_depth_ws_bytes(ctypes.byref(self.desc), ctypes.byref(f), ctypes.byref(b)),
+                   "hexa_moe_depth_ws_bytes")
+        self.fwd_bytes, self.bwd_bytes = int(f.value), int(b.value)
+
+
+def _event_array(events):
+    """ctypes array of hipEvent_t handles from torch.cuda.Event objects (each recorded once before, so that
+    its handle exists; None entries are skipped by the library), or (None, 0)."""
+    import ctypes
+    if not events:
+        return None, 0
+    arr = (ctypes.c_void_p * len(events))(*[None if e is None else e.cuda_event for e in events])
+    return arr, len(events)
+
+
+def moe_depth_forward(plan, x, wg, noise, fc1_w, fc1_b, fc2_w, fc2_b, logits, scores, idx, thr, stats, route_blob,
+                      y1, y2, y, ws, events=None):
+    import ctypes
+    _dev(x, wg, noise, fc1_w, fc1_b, fc2_w, fc2_b, idx, route_blob, y1, y2, y, ws)
+    ev, nev = _event_array(events)
+    rc = _lib.load().hexa_moe_depth_forward(ctypes.byref(plan.desc), _ptr(x), _ptr(wg), _ptr(noise), _ptr(fc1_w),
+                                            _ptr(fc1_b), _ptr(fc2_w), _ptr(fc2_b), _ptr(logits), _ptr(scores), _ptr(idx),
+                                            _ptr(thr), _ptr(stats), _ptr(route_blob), _ptr(y1), _ptr(y2), _ptr(y),
+                                            _ptr(ws), ws.numel() * ws.element_size(), ev, nev, _stream())
+    _lib.check(rc, "hexa_moe_depth_forward")
+
+
+def moe_depth_backward(plan, dy, grad_l_aux, x, wg, fc1_w, fc2_w, scores, idx, thr, stats, route_blob, y1, y2, dx, dwg,
+                       dw1, db1, dw2, db2, dy1, ws, events=None):
+    import ctypes
+    _dev(dy, grad_l_aux, x, wg, fc1_w, fc2_w, route_blob, y1, y2, dx, dwg, dw1, db1, dw2, db2, dy1, ws)
+    ev, nev = _event_array(events)
+    rc = _lib.load().hexa_moe_depth_backward(ctypes.byref(plan.desc), _ptr(dy), _ptr(grad_l_aux), _ptr(x), _ptr(wg),
+                                             _ptr(fc1_w), _ptr(fc2_w), _ptr(scores), _ptr(idx), _ptr(thr), _ptr(stats),
+                                             _ptr(route_blob), _ptr(y1), _ptr(y2), _ptr(dx), _ptr(dwg), _ptr(dw1),
+                                             _ptr(db1), _ptr(dw2), _ptr(db2), _ptr(dy1), _ptr(ws),
+                                             ws.numel() * ws.element_size(), ev, nev, _stream())
+    _lib.check(rc, "hexa_moe_depth_backward")

@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define HEXA_ABI_VERSION 5
+#define HEXA_ABI_VERSION 6
 
 /* element types */
 #define HEXA_F32 0
@@ -258,6 +258,59 @@ int hexa_router_forward_load_importance(float* scores, int32_t* idx, float* thr,
 int hexa_router_backward_load_importance(float* dlogits, const float* scores, const float* thr, const int32_t* idx,
                                          const float* g_importance, const float* g_load, const float* grad_l_aux,
                                          float sigma, int num_tokens, int num_experts, int top_k, void* stream);
+
+/* ---- one MoE depth per call ---------------------------------------------------------------------------
+ * hexa_moe_depth_forward / hexa_moe_depth_backward enqueue every kernel of one MoE depth -- the routing front
+ * end, the routing segment pass and the ten steps of the formula table with the exact-GELU activation -- from
+ * ONE call each, so a training step costs the host two library calls instead of two dozen.  They run the same
+ * kernels as the single-operator entry points above, in the same order, and give the same results.
+ * Replaces the bodies of MoE_Cascaded.forward's MoE branch (impls/cascaded_moe.py:508-568),
+ * FusedMoE_Shared_CudaCore.forward (impls/layers.py:99-277) and .backward (impls/layers.py:280-474).
+ *
+ * All sizes and element types travel in a descriptor.  act_dt is the type of x, y1, y2, y, dy, dy1 and dx; w_dt of
+ * fc1_w [E][hidden][d_in] and fc2_w [E][hidden][d_out] (act_dt or F32); b*_dt of the biases; g*_dt of the
+ * gradients (F32 or act_dt).  loss: 0 = GShard, 1 = load-importance (then sigma = gate_noise / E > 0). */
+typedef struct hexa_moe_depth_desc {
+    int32_t num_tokens, top_k, num_experts, d_in, hidden, d_out;
+    int32_t act_dt, w_dt, b1_dt, b2_dt, gw1_dt, gw2_dt, gb1_dt, gb2_dt;
+    int32_t loss;
+    float noise_scale; /* factor of `noise` in the logits (gate_noise / E while training, else 0) */
+    float sigma;       /* load-importance only */
+    int32_t reserved;
+} hexa_moe_depth_desc;
+
+/* Bytes of caller scratch the two calls need (either pointer may be NULL). */
+int hexa_moe_depth_ws_bytes(const hexa_moe_depth_desc* d, int64_t* forward_bytes, int64_t* backward_bytes);
+
+/* Forward.  With wg (fp32 [E][d_in]) the call starts at the gate: logits = x.wg^T (fp32), scores / idx / l_aux as
+ * hexa_router_forward or hexa_router_forward_load_importance (noise [T][E] fp32 or NULL); logits, scores [T][E],
+ * idx [T][k] int32, thr [T] (load-importance only, else NULL) and stats (GShard: me[E], ce[E], l_aux = 2E+1 floats;
+ * load-importance: importance, load, their two gradients, l_aux = 4E+1 floats) are outputs the backward needs.
+ * With wg == NULL the routing decision is the caller's: idx is read ([T][k] int32) and logits / scores / thr /
+ * stats / noise are ignored.
+ * Then: route = hexa_route_build(idx); y1 = x.W1^T + b1 and y2 = gelu(y1) ([k][T][hidden], saved for the backward);
+ * y [T][d_out] = sum over slots of y2.W2 + b2.  Biases may be NULL.
+ * events (may be NULL): 2*n caller-owned hipEvent_t handles; pair i is recorded on `stream` around major kernel i
+ * (0: fc1 + GELU, 1: fc2 and its slot sum), for callers that time kernels inside a step; NULL handles in the
+ * array are skipped. */
+int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* x, const float* wg, const float* noise,
+                           const void* fc1_w, const void* fc1_b, const void* fc2_w, const void* fc2_b, float* logits,
+                           float* scores, int32_t* idx, float* thr, float* stats, int32_t* route, void* y1, void* y2,
+                           void* y, void* ws, int64_t ws_bytes, void* const* events, int num_events, void* stream);
+
+/* Backward of the same depth from dy [T][d_out] and (with wg) the device scalar grad_l_aux (NULL: the auxiliary
+ * loss carries no gradient).  Results (each may be NULL to skip it): dx [T][d_in] = the expert path's input
+ * gradient plus, with wg, the gate path's; dwg [E][d_in] fp32; dw1 [E][hidden][d_in], db1 [E][hidden],
+ * dw2 [E][hidden][d_out], db2 [E][d_out].  dy1 is caller memory for the hidden gradient ([k][T][hidden] of act_dt);
+ * its contents after the call are dy1 = (dy.W2^T) * gelu'(y1).
+ * events: pairs around (0) the dy1 kernel with its bias-gradient sums, (1) the dx kernel and its slot sum,
+ * (2) ESTMM dW2, (3) ESTMM dW1. */
+int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void* dy, const float* grad_l_aux, const void* x,
+                            const float* wg, const void* fc1_w, const void* fc2_w, const float* scores,
+                            const int32_t* idx, const float* thr, const float* stats, const int32_t* route,
+                            const void* y1, const void* y2, void* dx, float* dwg, void* dw1, void* db1, void* dw2,
+                            void* db2, void* dy1, void* ws, int64_t ws_bytes, void* const* events, int num_events,
+                            void* stream);
 
 const char* hexa_last_error(void);
 int hexa_abi_version(void);

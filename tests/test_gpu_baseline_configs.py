@@ -54,14 +54,15 @@ def test_esmm_swin_stage3_shape(dev):
     assert_close(got_t, want, TOL[BF16], "esmm [E,out,in]")
 
 
-def test_layer_fwd_bwd_T4608_d768(dev):
+@pytest.mark.parametrize("act", [F.gelu, lambda t: F.gelu(t)], ids=["fused_gelu", "generic_activation"])
+def test_layer_fwd_bwd_T4608_d768(dev, act):
     from hexa_moe import moe as hmoe
     T, d, E, k = 4608, 768, 32, 1
     print(f"config layer T={T} d={d} h={4 * d} E={E} k={k} bf16 seed=1236", flush=True)
     torch.manual_seed(1236)
     m = hmoe.MoE_Cascaded(gate_type={'type': 'top', 'k': k, 'gate_noise': 0.0, 'fp32_gate': True},
                           model_dim_list=[d], moe_idx_list=[0], mlp_ratio=4, num_global_experts=E, total_depth=1,
-                          data_centric=True, mlp_fc1_bias=True, mlp_fc2_bias=True, activation_fn=lambda t: F.gelu(t))
+                          data_centric=True, mlp_fc1_bias=True, mlp_fc2_bias=True, activation_fn=act)
     g = gen(1236)
     for name, p in m.named_parameters():
         fan_in = p.shape[-1] if name.startswith(("batched_fc1_w", "gates")) else p.shape[-2] if p.dim() > 1 else p.shape[-1]
@@ -71,7 +72,7 @@ def test_layer_fwd_bwd_T4608_d768(dev):
     dy = torch.randn(T, d, generator=g).to(BF16)
     xd = x.to(dev).requires_grad_(True)
     y, _ = m(0, xd)
-    routing = m.dispatch_params.indices_.cpu()
+    routing = m.dispatch_params.routing_.cpu()
     y.backward(dy.to(dev))
     torch.cuda.synchronize()
     W1, W2 = m.batched_fc1_w[0].detach().cpu().float(), m.batched_fc2_w[0].detach().cpu().float()

@@ -45,12 +45,17 @@ def test_readme_config_fp32(dev):
     x = x0.to(dev).requires_grad_(True)
     h = x
     captured = []
+    dense = []
     aux = 0
     for depth in range(4):
         h_in = h
         h, l_aux = m(depth, h)
+        if depth in (0, 1):
+            assert l_aux == 0            # a dense depth has no auxiliary loss (cascaded_moe.py:506)
+            dense.append((depth, h_in, h))
+            h.retain_grad(); h_in.retain_grad()
         if depth in (2, 3):
-            captured.append((depth, h_in, m.dispatch_params.indices_.clone(), h))
+            captured.append((depth, h_in, m.dispatch_params.routing_.clone(), h))
             h.retain_grad(); h_in.retain_grad()
             aux = aux + l_aux
     (h.sum() + aux).backward()
@@ -68,21 +73,33 @@ def test_readme_config_fp32(dev):
         if depth == 3:   # h_in.grad of depth 3 is purely the layer's dx (+ the gate's aux-loss path)
             gate_free = h_in.grad.detach().cpu().double() - dx
             assert gate_free.abs().max() < 1e-2   # what is left is the small l_aux gradient through the gate
+    # the dense depths (MLP_Implement) against the oracle's dense FFN, differentiated by autograd in fp64
+    for depth, h_in, h_out in dense:
+        i = [d_ for d_ in range(4) if d_ not in (2, 3)].index(depth)
+        prm = [m.mlp_fc1_w[i], m.mlp_fc2_w[i], m.mlp_fc1_b[i], m.mlp_fc2_b[i]]
+        ref_p = [q.detach().cpu().double().requires_grad_(True) for q in prm]
+        xin = h_in.detach().cpu().double().requires_grad_(True)
+        y_ref = O.dense_mlp_forward(xin, ref_p[0], ref_p[1], ref_p[2], ref_p[3], F.gelu)
+        y_ref.backward(h_out.grad.cpu().double())
+        assert_close(h_out.detach(), y_ref.detach(), 1e-5, f"dense y depth {depth}")
+        assert_close(h_in.grad, xin.grad, 1e-5, f"dense dx depth {depth}")
+        for q, r, name in zip(prm, ref_p, ["fc1_w", "fc2_w", "fc1_bias", "fc2_bias"]):
+            assert_close(q.grad, r.grad, 1e-5, f"dense {name} depth {depth}")
     assert x.grad is not None and m.gates[0].wg.weight.grad is not None
-    assert m.mlp_fc1_w[0].grad is not None
 
 
 @pytest.mark.parametrize("dtype,k,bias", [(torch.float32, 2, True), (torch.bfloat16, 1, True), (torch.bfloat16, 2, False),
                                           (torch.float16, 2, True)])
-def test_single_depth_against_oracle(dev, dtype, k, bias):
+@pytest.mark.parametrize("act", [F.gelu, None], ids=["fused_gelu", "generic_activation"])
+def test_single_depth_against_oracle(dev, dtype, k, bias, act):
     E, d, T = 16, 256, 3000
-    m = _module([d], [0], E=E, k=k, bias=bias, noise=0.0).to(dev).to(dtype).eval()
+    m = _module([d], [0], E=E, k=k, bias=bias, noise=0.0, act=act).to(dev).to(dtype).eval()
     g = torch.Generator().manual_seed(7)
     x = torch.randn(T, d, generator=g).to(dtype)
     dy = torch.randn(T, d, generator=g).to(dtype)
     xd = x.to(dev).requires_grad_(True)
     y, l_aux = m(0, xd)
-    routing = m.dispatch_params.indices_.cpu()
+    routing = m.dispatch_params.routing_.cpu()
     y.backward(dy.to(dev))
     torch.cuda.synchronize()
     assert y.dtype == dtype and l_aux.dim() == 0
@@ -138,7 +155,7 @@ def test_stochastic_activation_uses_one_mask(dev):
     torch.cuda.synchronize()
     assert len(masks) == 1, "the activation must be evaluated exactly once per forward+backward"
     mk = masks[0].cpu().double()
-    routing = m.dispatch_params.indices_.cpu()
+    routing = m.dispatch_params.routing_.cpu()
     y_ref, (dx, dW1, dW2, db1, db2) = _oracle_depth(m, 0, x.detach().cpu(), routing, dy.cpu(), lambda t: F.gelu(t) * mk, torch.float64)
     assert_close(y.detach(), y_ref, 1e-5, "y")
     assert_close(x.grad, dx, 1e-5, "dx")
@@ -157,7 +174,7 @@ def test_autocast_bf16_with_fp32_master_weights(dev):
     h.retain_grad()
     y.backward(dy)
     torch.cuda.synchronize()
-    routing = m.dispatch_params.indices_.cpu()
+    routing = m.dispatch_params.routing_.cpu()
     hb = h.detach().to(torch.bfloat16).float().cpu()
     W1 = m.batched_fc1_w[0].detach().to(torch.bfloat16).float().cpu()
     W2 = m.batched_fc2_w[0].detach().to(torch.bfloat16).float().cpu()
@@ -191,3 +208,63 @@ def test_route_pool_is_reused_across_steps_and_survives_pending_backward(dev):
         before = pool._slots[1][0]
         m(1, x)
         assert pool._slots[1][0] is before
+
+
+@pytest.mark.parametrize("loss", ["gshard", "load_importance"])
+def test_nan_token_row_stays_routed_and_propagates(dev, loss):
+    """A token whose features are NaN gets NaN gate logits.  torch.topk ranks NaN largest and still returns
+    valid expert ids, so the reference routes the token, its output row is NaN and the auxiliary loss is NaN
+    (which is what an AMP scaler looks for).  The fused router must not drop the token or leave its rows
+    unwritten: valid ids, NaN in y and dx for that token only, NaN l_aux."""
+    E, d, T, k = 8, 128, 700, 2
+    m = _module([d], [0], E=E, k=k, act=F.gelu, noise=1.0).to(dev).train()
+    m.is_gshard_loss = loss == "gshard"
+    x = torch.randn(T, d, generator=torch.Generator().manual_seed(3))
+    bad = 123
+    x[bad] = float("nan")
+    xd = x.to(dev).requires_grad_(True)
+    y, l_aux = m(0, xd)
+    idx = m.dispatch_params.routing_
+    idx = idx if torch.is_tensor(idx) else torch.stack(list(idx), 1)
+    y.sum().backward()
+    torch.cuda.synchronize()
+    assert int(idx.min()) >= 0 and int(idx.max()) < E
+    assert torch.isnan(y[bad]).all() and torch.isnan(xd.grad[bad]).all()
+    keep = torch.ones(T, dtype=torch.bool)
+    keep[bad] = False
+    assert torch.isfinite(y[keep.to(dev)]).all() and torch.isfinite(xd.grad[keep.to(dev)]).all()
+    assert torch.isnan(l_aux)
+
+
+@pytest.mark.parametrize("loss", ["gshard", "load_importance"])
+@pytest.mark.parametrize("dtype,k,bias", [(torch.float32, 1, True), (torch.bfloat16, 2, True), (torch.float16, 2, False),
+                                          (torch.bfloat16, 1, True)])
+def test_depth_call_equals_operator_by_operator(dev, dtype, k, bias, loss):
+    """hexa_moe_depth_forward / _backward (one library call per direction) run the same kernels in the same
+    order as the per-operator path: same routing, identical y, l_aux and parameter gradients; dx differs only
+    by where the gate path's share is added (inside the slot sum instead of a separate addition)."""
+    E, d, T = 16, 256, 2500
+    m = _module([d], [0], E=E, k=k, bias=bias, act=F.gelu, noise=1.0).to(dev).to(dtype).eval()
+    m.gates[0].wg.weight.data = m.gates[0].wg.weight.data.float()
+    m.is_gshard_loss = loss == "gshard"
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(T, d, generator=g).to(dtype).to(dev)
+    dy = torch.randn(T, d, generator=g).to(dtype).to(dev)
+    res = []
+    for fused_depth in (True, False):
+        m.fused_depth = fused_depth
+        m.zero_grad(set_to_none=True)
+        xi = x.clone().requires_grad_(True)
+        y, l_aux = m(0, xi)
+        torch.autograd.backward([y, l_aux], [dy, torch.full((), 3.0, device=dev)])
+        torch.cuda.synchronize()
+        assert len(m.dispatch_params.indices_) == k and m.dispatch_params.indices_[0].dtype == torch.int32
+        grads = [p.grad.clone() for p in (m.gates[0].wg.weight, m.batched_fc1_w[0], m.batched_fc2_w[0])]
+        if bias:
+            grads += [m.batched_fc1_bias[0].grad.clone(), m.batched_fc2_bias[0].grad.clone()]
+        res.append((m.dispatch_params.routing_.clone().long(), y.detach().clone(), l_aux.detach().clone(), xi.grad.clone(), grads))
+    (ra, ya, la, dxa, ga), (rb, yb, lb, dxb, gb) = res
+    assert torch.equal(ra, rb) and torch.equal(ya, yb) and torch.equal(la, lb)
+    for u, v in zip(ga, gb):
+        assert torch.equal(u, v)
+    assert_close(dxa, dxb, 1e-6 if dtype == torch.float32 else 1e-2, "dx")

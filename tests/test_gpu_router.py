@@ -155,7 +155,7 @@ def test_module_fused_and_framework_routing_agree(dev, dtype, gshard):
         xi = x.clone().requires_grad_(True)
         y, l_aux = m(0, xi)
         (y.float().sum() + 10.0 * l_aux).backward()
-        res.append((m.dispatch_params.indices_.clone().long(), l_aux.detach(), y.detach(), xi.grad, m.gates[0].wg.weight.grad.clone()))
+        res.append((m.dispatch_params.routing_.clone().long(), l_aux.detach(), y.detach(), xi.grad, m.gates[0].wg.weight.grad.clone()))
     torch.cuda.synchronize()
     a, b = res
     assert torch.equal(a[0], b[0]), "same expert choices"

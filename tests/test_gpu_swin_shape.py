@@ -29,7 +29,7 @@ class Capture:
     def __call__(self, depth, ffn_in, ffn_out):
         if depth in self.depths:
             ffn_out.retain_grad()
-            self.seen[depth] = (ffn_in.detach(), self.model.cascaded_moe.dispatch_params.indices_.clone(), ffn_out)
+            self.seen[depth] = (ffn_in.detach(), self.model.cascaded_moe.dispatch_params.routing_.clone(), ffn_out)
 
 
 def _check_depth(model, depth, seen, tol, rd):

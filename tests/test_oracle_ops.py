@@ -179,3 +179,44 @@ def test_load_importance_loss_closed_forms():
     imp = torch.tensor([float(T), 0, 0, 0]); load = torch.tensor([float(T), 0, 0, 0])
     want = (imp.var() / imp.mean() ** 2 + load.var() / load.mean() ** 2) / 2
     assert abs(float(O.load_importance_loss(scores, thr, E, 1e-3)) - float(want)) < 1e-4
+
+
+def test_load_importance_loss_sigma_is_gate_noise_over_experts():
+    """The width of the normal CDF is gate_noise / E (impls/losses.py:27-33: Normal(0, gate_noise / E)).
+    An independent evaluation with torch.special.ndtr, in the steep regime (scores within a few sigma of
+    the threshold), differs from one with sigma = gate_noise by far more than the tolerance, so a dropped
+    `/ E` in the oracle fails here."""
+    g = torch.Generator().manual_seed(11)
+    T, E, noise = 512, 8, 0.16          # sigma = 0.02
+    scores = torch.softmax(0.3 * torch.randn(T, E, generator=g), 1).double()
+    thr = scores.mean(1, keepdim=True) + 0.01 * torch.randn(T, 1, generator=g).double()
+
+    def independent(sigma):
+        load = torch.special.ndtr((scores - thr) / sigma).sum(0)
+        imp = scores.sum(0)
+        cv2 = lambda v: v.var(unbiased=True) / (v.mean() ** 2 + 1e-10)   # noqa: E731
+        return float((cv2(imp) + cv2(load)) / 2)
+
+    got = float(O.load_importance_loss(scores.float(), thr.float(), E, noise))
+    assert abs(got - independent(noise / E)) < 1e-5 * max(1.0, abs(got))
+    assert abs(independent(noise) - independent(noise / E)) > 5e-4      # 50x the tolerance above: the scales are far apart
+
+
+def test_nan_token_row_in_the_oracle():
+    """Pins what the GPU test of a NaN token row expects: softmax of a row with a NaN is all NaN, torch.topk
+    still returns ids in [0, E), the token stays in its experts' lists, and its output row is NaN while every
+    other row is finite."""
+    g = torch.Generator().manual_seed(5)
+    T, d, h, E, k = 64, 16, 32, 4, 2
+    x = torch.randn(T, d, generator=g)
+    x[7] = float("nan")
+    wg = torch.randn(E, d, generator=g)
+    scores, idx = O.route_top_k(x @ wg.t(), k)
+    assert torch.isnan(scores[7]).all() and int(idx.min()) >= 0 and int(idx.max()) < E
+    counts, offsets, token_ids = O.route_build(idx, E)
+    assert int(counts.sum()) == T * k and (token_ids == 7).sum() == k
+    W1, W2 = torch.randn(E, h, d, generator=g), torch.randn(E, h, d, generator=g)
+    y, _, _ = O.moe_ffn_forward(x, W1, W2, None, None, idx, F.gelu)
+    assert torch.isnan(y[7]).all()
+    keep = torch.ones(T, dtype=torch.bool); keep[7] = False
+    assert torch.isfinite(y[keep]).all()

@@ -20,7 +20,7 @@ void set_error(const char* fmt, ...) {
 namespace {
 struct OptEntry { const char* name; const char* env; int value; bool loaded; };
 OptEntry g_opts[OPT_COUNT] = {
-    {"tile", "HEXA_MOE_TILE", 0, false},          {"persist", "HEXA_MOE_PERSIST", 0, false},
+    {"tile", "HEXA_MOE_TILE", 0, false},          {"pipe", "HEXA_MOE_PIPE", 0, false},
     {"general_kernels", "HEXA_MOE_GENERAL_KERNELS", 0, false}, {"esmm_map", "HEXA_ESMM_MAP", 0, false},
     {"esmm_group", "HEXA_ESMM_GROUP", 0, false},  {"estmm_group", "HEXA_ESTMM_GROUP", 0, false},
     {"esmm_stream", "HEXA_ESMM_STREAM", 0, false}, {"route_kernels", "HEXA_ROUTE_KERNELS", 0, false},

@@ -39,6 +39,8 @@ using CfgS3 = Cfg<2, 2, 2, 2, 3, 3>;  // 128 x 128, 3 stages, 3 workgroups per C
 using CfgS64 = Cfg<2, 2, 2, 2, 2, 2, 64>;  // 128 x 128, 64 contraction indices per stage, 2 stages
 using CfgL64 = Cfg<4, 2, 2, 2, 2, 4, 64>;  // 256 x 128, 8 wavefronts, 64 per stage, 2 stages
 using CfgW = Cfg<2, 4, 2, 3, 3, 2>;   // 128 x 384, 8 wavefronts of 64x96: one tile spans a 384-wide result
+using CfgS64W = Cfg<2, 4, 2, 1, 2, 4, 64>;   // 128 x 128, 8 wavefronts of 64x32, 64 per stage, 2 stages, 2 workgroups per CU
+using CfgS64H = Cfg<4, 2, 1, 2, 2, 4, 64>;   // 128 x 128, 8 wavefronts of 32x64, 64 per stage, 2 stages, 2 workgroups per CU
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
@@ -67,6 +69,16 @@ typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 // One wavefront copy: every lane fetches 16 bytes from `src`; lane i lands at lds_base + 16*i.
 __device__ __forceinline__ void dma16(const void* src, char* lds_base) {
     __builtin_amdgcn_global_load_lds((glb_ptr_t)src, (lds_ptr_t)lds_base, 16, 0, 0);
+}
+
+// 16-byte store; `streaming` marks the line as not worth keeping in the caches (results that are much
+// larger than the L2 would otherwise push the weights and token rows out of it)
+__device__ __forceinline__ void store16(uint4* dst, uint4 v, bool streaming) {
+    typedef __attribute__((ext_vector_type(4))) unsigned u4;
+    u4 w;
+    w.x = v.x; w.y = v.y; w.z = v.z; w.w = v.w;
+    if (streaming) __builtin_nontemporal_store(w, reinterpret_cast<u4*>(dst));
+    else *reinterpret_cast<u4*>(dst) = w;
 }
 
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
@@ -226,23 +238,36 @@ template <typename TC> __device__ __forceinline__ uint2 pack4(float a, float b, 
     return o;
 }
 
-// GELU (erf form) with erf from Abramowitz & Stegun 7.1.26 (|error| < 1.5e-7): one exp2, one hardware
-// reciprocal and a degree-5 polynomial instead of the library erff (whose division alone is a dozen
-// instructions).  The epilogue's arithmetic is not free here: a wavefront's VALU instruction occupies
-// its SIMD for 4 cycles (16 for the transcendental ones), and at a contraction length of a few hundred
-// a tile's epilogue costs about as many SIMD cycles as its MFMAs.  Used where the result is rounded to
-// 16 bits (or compared at 2e-2); the fp32 kernels keep erff.  (An 8-term odd polynomial for erf,
-// FMAs only, was measured too: 5 % faster on the fused fc1 launch at 1.5e-4 error -- not taken.)
-__device__ __forceinline__ float gelu_fast(float x) {
-    const float z = fabsf(x) * 0.70710678118654752440f;
-    const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
-    const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
-    const float erf_abs = 1.0f - poly * __expf(-z * z);
-    const float erf_x = copysignf(erf_abs, x);
-    return 0.5f * x * (1.0f + erf_x);
+// GELU (erf form) for results that are rounded to 16 bits (or compared at 2e-2), without a transcendental
+// instruction.  The epilogue's arithmetic is not free here: a wavefront's VALU instruction occupies its SIMD
+// for 4 cycles (16 for a transcendental one), and at a contraction length of a few hundred a tile's GELU costs
+// about as many SIMD cycles as its MFMAs.  erf(z) = z * Q(z^2) on |z| <= 3 (clamped beyond: erf(3) = 1 - 2e-5),
+// Q of degree 8 fitted to |error| < 3e-5 in fp32 -- bf16 / fp16 round at 4e-3 / 5e-4 relative --: 14 VALU
+// operations per element against 12 + two transcendental ones (= 20 issue slots) for the Abramowitz-Stegun
+// form with exp and a reciprocal that was used before.  The fp32 kernels keep erff.
+__device__ __forceinline__ float erf_poly(float z) {
+    const float zc = __builtin_amdgcn_fmed3f(z, -3.0f, 3.0f);
+    const float s = zc * zc;
+    float q = 4.074186864e-08f;
+    q = fmaf(q, s, -1.944813793e-06f);
+    q = fmaf(q, s, 4.106038601e-05f);
+    q = fmaf(q, s, -5.110357344e-04f);
+    q = fmaf(q, s, 4.235422156e-03f);
+    q = fmaf(q, s, -2.510284743e-02f);
+    q = fmaf(q, s, 1.110793160e-01f);
+    q = fmaf(q, s, -3.753148625e-01f);
+    q = fmaf(q, s, 1.128268422e+00f);
+    return zc * q;
 }
+__device__ __forceinline__ float gelu_poly(float x) {
+    const float hx = 0.5f * x;
+    return fmaf(hx, erf_poly(x * 0.70710678118654752440f), hx);
+}
+__device__ __forceinline__ float gelu_fast(float x) { return gelu_poly(x); }
 
-// gelu'(x) = Phi(x) + x*phi(x) with the same erf approximation (shares its exponential)
+// gelu'(x) = Phi(x) + x * phi(x) needs exp(-x^2 / 2) anyway, so erf comes from Abramowitz & Stegun 7.1.26
+// (|error| < 1.5e-7), which shares that exponential: one exp2, one hardware reciprocal and a degree-5 polynomial
+// (measured against the polynomial erf above plus a separate exponential: 127 vs 140 us for the backward launch).
 __device__ __forceinline__ float gelu_grad_fast(float x) {
     const float z = fabsf(x) * 0.70710678118654752440f;
     const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
@@ -251,6 +276,7 @@ __device__ __forceinline__ float gelu_grad_fast(float x) {
     const float erf_x = copysignf(1.0f - poly * ex, x);
     return 0.5f * (1.0f + erf_x) + x * 0.39894228040143267794f * ex;
 }
+__device__ __forceinline__ float gelu_grad_poly(float x) { return gelu_grad_fast(x); }
 
 // ------------------------------------------------------------------------------------------------
 // ESMM

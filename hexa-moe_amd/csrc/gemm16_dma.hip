@@ -32,16 +32,6 @@
 namespace hexa {
 namespace {
 
-// 16-byte store; `streaming` marks the line as not worth keeping in the caches (results that are much
-// larger than the L2 would otherwise push the weights and token rows out of it)
-__device__ __forceinline__ void store16(uint4* dst, uint4 v, bool streaming) {
-    typedef __attribute__((ext_vector_type(4))) unsigned u4;
-    u4 w;
-    w.x = v.x; w.y = v.y; w.z = v.z; w.w = v.w;
-    if (streaming) __builtin_nontemporal_store(w, reinterpret_cast<u4*>(dst));
-    else *reinterpret_cast<u4*>(dst) = w;
-}
-
 template <typename TC, bool W_IN_OUT, bool OUT32, typename C>
 __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
     constexpr int BM = C::BM, BN = C::BN, STAGES = C::STAGES, NW = C::NW, BK = C::BKC;
@@ -769,12 +759,7 @@ int launch_esmm_dma_c(const EsmmArgs& a, bool large, hipStream_t st) {
         if (rc) return rc;
     }
     if (p.ws) return launch_sum_slots(a.out, a.slot_ws, (int64_t)a.r.T * a.out_dim, a.r.k - 1, a.out_dt, st, a.sum_extra);
-    if (a.colsum) {
-        hipLaunchKernelGGL(esmm_colsum_fold_kernel, dim3(div_up(a.out_dim, 256), a.r.E), dim3(256), 0, st, a.db, a.colsum,
-                           a.r.offsets, a.r.E, p.mt_ub, large ? HEXA_TILE_ROWS_L : HEXA_TILE_ROWS, p.ntn, C::BN, a.out_dim,
-                           a.r.k, a.db_dt, a.db_accumulate);
-        HEXA_CHECK_LAUNCH("esmm_colsum_fold");
-    }
+    if (a.colsum) return launch_colsum_fold(a, p.mt_ub, large ? HEXA_TILE_ROWS_L : HEXA_TILE_ROWS, p.ntn, C::BN, st);
     return HEXA_OK;
 }
 
@@ -791,6 +776,13 @@ int pick_esmm_tile(long rows, int cols, int in_dim) {
 }
 
 }  // namespace
+
+int launch_colsum_fold(const EsmmArgs& a, int mt_ub, int tile_rows, int ntn, int bn, hipStream_t st) {
+    hipLaunchKernelGGL(esmm_colsum_fold_kernel, dim3(div_up(a.out_dim, 256), a.r.E), dim3(256), 0, st, a.db, a.colsum, a.r.offsets,
+                       a.r.E, mt_ub, tile_rows, ntn, bn, a.out_dim, a.r.k, a.db_dt, a.db_accumulate);
+    HEXA_CHECK_LAUNCH("esmm_colsum_fold");
+    return HEXA_OK;
+}
 
 int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, hipStream_t st) {
     if (r.E > 4096) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "estmm plan: more than 4096 experts");
@@ -835,19 +827,15 @@ int launch_estmm16_dma(const EstmmArgs& a, hipStream_t st) {
     }
 }
 
-// HEXA_MOE_PERSIST=1 selects the persistent-workgroup ESMM kernels (read once).  They are parity-
-// tested but not the default: on the shapes measured so far the one-tile-per-workgroup kernels win.
-static bool persist_enabled() { return option(OPT_PERSIST) == 1; }
-
-// The column sums ride on the store loop of the per-slot, 16-bit-result kernels (not the persistent one, not
-// the 128x384 tile, whose rows have 48 pieces).
+// The column sums ride on the store loop of the per-slot, 16-bit-result kernels (not
+// the 128x384 tile, whose rows have 48 pieces); the pipelined kernel has its own.
 bool esmm16_dma_colsum_supported(const EsmmArgs& a) {
-    return esmm16_dma_supported(a) && a.out_dt == a.x_dt && a.out_per_slot && a.r.k <= 8 && forced_tile() != 7 &&
-           !(persist_enabled() && esmm16_persist_supported(a));
+    if (option(OPT_PIPE) == 1 && esmm16_pipe_supported(a)) return a.out_per_slot && a.r.k <= 8;
+    return esmm16_dma_supported(a) && a.out_dt == a.x_dt && a.out_per_slot && a.r.k <= 8 && forced_tile() != 7;
 }
 
 int launch_esmm16_dma(const EsmmArgs& a, hipStream_t st) {
-    if (persist_enabled() && esmm16_persist_supported(a)) return launch_esmm16_persist(a, forced_tile(), st);
+    if (option(OPT_PIPE) == 1 && esmm16_pipe_supported(a)) return launch_esmm16_pipe(a, st);
     if (forced_tile() == 7) return launch_esmm_dma_c<CfgW>(a, false, st);
     switch (pick_esmm_tile((long)a.r.T * a.r.k, a.out_dim, a.in_dim)) {
         case 2: return launch_esmm_dma_c<CfgL>(a, true, st);
@@ -858,6 +846,8 @@ int launch_esmm16_dma(const EsmmArgs& a, hipStream_t st) {
         case 8: return launch_esmm_dma_c<CfgS2>(a, false, st);
         case 10: return (a.in_dim % 64) ? launch_esmm_dma_c<CfgS>(a, false, st) : launch_esmm_dma_c<CfgS64>(a, false, st);
         case 11: return (a.in_dim % 64) ? launch_esmm_dma_c<CfgL>(a, true, st) : launch_esmm_dma_c<CfgL64>(a, true, st);
+        case 12: return (a.in_dim % 64) ? launch_esmm_dma_c<CfgS>(a, false, st) : launch_esmm_dma_c<CfgS64W>(a, false, st);
+        case 13: return (a.in_dim % 64) ? launch_esmm_dma_c<CfgS>(a, false, st) : launch_esmm_dma_c<CfgS64H>(a, false, st);
         case 9: return launch_esmm_dma_c<CfgS3>(a, false, st);
         default: return launch_esmm_dma_c<CfgS>(a, false, st);
     }

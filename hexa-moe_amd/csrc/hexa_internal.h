@@ -87,7 +87,7 @@ int launch_esmm32(const EsmmArgs& a, hipStream_t s);
 // can be changed at run time with hexa_set_option.
 enum Opt {
     OPT_TILE,           // HEXA_MOE_TILE: tile configuration of the 16-bit fast path (see gemm16_dma.hip)
-    OPT_PERSIST,        // HEXA_MOE_PERSIST: 1 = persistent-workgroup ESMM kernels
+    OPT_PIPE,           // HEXA_MOE_PIPE: 1 = pipelined persistent ESMM kernel (multiply, copy and store wavefronts side by side)
     OPT_GENERAL,        // HEXA_MOE_GENERAL_KERNELS: 1 = general 16-bit kernels instead of the fast path
     OPT_ESMM_MAP,       // HEXA_ESMM_MAP: 2 = runs of tiles per XCD instead of one contiguous eighth of the tiles per XCD
     OPT_ESMM_GROUP,     // HEXA_ESMM_GROUP: row tiles per XCD run
@@ -100,9 +100,10 @@ int option(int id);
 
 bool esmm16_dma_supported(const EsmmArgs& a);
 bool esmm16_dma_colsum_supported(const EsmmArgs& a);
-bool esmm16_persist_supported(const EsmmArgs& a);
+bool esmm16_pipe_supported(const EsmmArgs& a);
+int launch_esmm16_pipe(const EsmmArgs& a, hipStream_t st);
+int launch_colsum_fold(const EsmmArgs& a, int mt_ub, int tile_rows, int ntn, int bn, hipStream_t st);
 int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, hipStream_t st);
-int launch_esmm16_persist(const EsmmArgs& a, int tile, hipStream_t st);
 int launch_esmm16_dma(const EsmmArgs& a, hipStream_t s);
 bool dma_path_enabled();
 bool estmm16_dma_supported(const EstmmArgs& a);

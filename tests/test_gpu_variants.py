@@ -1,4 +1,4 @@
-"""Every kernel variant of the 16-bit fast path (tile shapes, persistent workgroups, tile-to-XCD mapping,
+"""Every kernel variant of the 16-bit fast path (tile shapes, the pipelined persistent kernel, tile-to-XCD mapping,
 general kernels) must give the same results: the operators are run under each setting of the library's
 tuning knobs and compared with the CPU oracle."""
 import pytest
@@ -10,10 +10,10 @@ from oracle import hexa_oracle as O
 pytestmark = pytest.mark.gpu
 
 SETTINGS = [{"tile": t} for t in range(1, 12)] + [
-    {"persist": 1}, {"persist": 1, "tile": 2}, {"persist": 1, "tile": 3},
+    {"pipe": 1}, {"tile": 12}, {"tile": 13},
     {"esmm_map": 2}, {"esmm_map": 2, "esmm_group": 16}, {"estmm_group": 4}, {"estmm_group": 12}, {"esmm_stream": 1}, {"general_kernels": 1},
 ]
-ALL = ("tile", "persist", "esmm_map", "esmm_group", "estmm_group", "esmm_stream", "general_kernels")
+ALL = ("tile", "pipe", "esmm_map", "esmm_group", "estmm_group", "esmm_stream", "general_kernels")
 
 
 @pytest.fixture
@@ -52,6 +52,9 @@ def test_variant(dev, knobs, cfg, dtype):
     (want_g,) = torch.autograd.grad(torch.nn.functional.gelu(y1r), y1r, lin.double())
     got = ops.esmm(x.to(dev), Wt, None, route, False, _lib.HEXA_W_OUT_IN, gelu_bwd_of=y1)
     assert_close(got, want_g, TOL[dtype], "esmm * gelu'")
+    got, db = ops.esmm_gelu_bwd_ess(x.to(dev), Wt, route, _lib.HEXA_W_OUT_IN, y1)
+    assert_close(got, want_g, TOL[dtype], "esmm * gelu' (with column sums)")
+    assert_close(db, O.ess(got.float().cpu(), token_ids, offsets, True, E), 1e-5, "column sums of the stored result")
     # sum over slots (per-slot operand), accumulating
     xs = torch.randn(k, T, d_out, generator=g).to(dtype)
     W2 = ((torch.rand(E, d_out, d_in, generator=g) * 2 - 1) / d_out ** 0.5).to(dtype)

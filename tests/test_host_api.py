@@ -162,3 +162,19 @@ def test_skip_moe_env(monkeypatch):
     x = torch.randn(8, 128)
     y, l = m(2, x)
     assert y is x and l is None
+
+
+def test_triton_sibling_surface_signatures():
+    """hexa_moe.kernels exports counter / ESMM / es_fused with the argument lists of
+    hexa_moe_triton/hexa_moe/kernels (basics.py:89, esmm.py:249, fused.py:382)."""
+    import inspect
+    from hexa_moe import kernels
+    from hexa_moe.kernels import constant
+    assert constant.MAX_TOKEN_CHUNK == 16
+    assert list(inspect.signature(kernels.counter).parameters) == ["routing", "num_exps"]
+    assert list(inspect.signature(kernels.ESMM).parameters) == ["toks", "w", "b", "tok_ids_list", "exp_ids_list"]
+    assert list(inspect.signature(kernels.es_fused).parameters) == ["tok1", "tok2", "w", "tok_ids_list", "exp_ids_list",
+                                                                    "exp_start_list", "num_exps", "bias"]
+    import torch
+    with __import__("pytest").raises(RuntimeError):
+        kernels.counter(torch.zeros(8, dtype=torch.int32), 4)       # CPU tensors are rejected: no fallback

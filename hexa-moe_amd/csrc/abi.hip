@@ -181,7 +181,8 @@ extern "C" int hexa_ess_noalloc(void* db, const void* dy, const int32_t* route, 
 extern "C" int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y, const void* w, const void* x,
                                const int32_t* route, int m2s, int accumulate, int T, int k, int in_dim, int out_dim,
                                int E, int act_dt, int w_dt, int jx_dt, int jw_dt, int jb_dt, void* slot_ws,
-                               void* stream) {
+                               const int32_t* plan, int max_slots, float* estmm_scratch, float* ess_ws,
+                               int64_t ess_ws_floats, void* stream) {
     if (!j_x || !j_w || !j_y || !w || !x || !route) HEXA_FAIL(HEXA_ERR_ARG, "hexa_fused_grad: null pointer");
     // ESMM task: j_x = j_y . w[e] with w [E][out][in] read as an [E][in'=out][out'=in] weight; the
     // slot layout is the mirror image of the forward's (shared j_y -> per-slot j_x and vice versa).
@@ -190,9 +191,11 @@ extern "C" int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y,
     if (rc) return rc;
     // ESTMM task: j_w[e][out][in] = sum j_y^T x
     rc = hexa_estmm(j_w, j_y, x, route, m2s ? 1 : 0, m2s ? 0 : 1, accumulate, T, k, out_dim, in_dim, E, act_dt, jw_dt,
-                    nullptr, 0, nullptr, stream);
+                    plan, max_slots, estmm_scratch, stream);
     if (rc) return rc;
-    if (j_b) rc = hexa_ess(j_b, j_y, route, m2s ? 1 : 0, accumulate, T, k, out_dim, E, act_dt, jb_dt, nullptr, 0, stream);
+    if (j_b)
+        rc = hexa_ess(j_b, j_y, route, m2s ? 1 : 0, accumulate, T, k, out_dim, E, act_dt, jb_dt, ess_ws,
+                      ess_ws ? ess_ws_floats : 0, stream);
     return rc;
 }
 

@@ -96,7 +96,7 @@ struct PipeK {
     int wg_per_xcd;       // workgroups per XCD (grid = 8 * wg_per_xcd)
 };
 
-constexpr int PIPE_COPY_WAVES = 4, PIPE_STORE_WAVES = 4;
+constexpr int PIPE_COPY_WAVES = 8, PIPE_STORE_WAVES = 4;
 
 template <typename C> struct PipeLds {
     static constexpr int CP = C::BN * 2 + 16;                 // pitch of a staged 16-bit result row

@@ -47,7 +47,8 @@ SIGNATURES = {
     "hexa_estmm_plan": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
     "hexa_ess": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
     "hexa_ess_noalloc": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
-    "hexa_fused_grad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp]),
+    "hexa_fused_grad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
+                             _vp, _i, _vp, _vp, _i64, _vp]),
     "hexa_gelu_bwd": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),
     "hexa_esmm_ess_ws_floats": (_i, [_i, _i, _i, _i, ctypes.POINTER(_i64)]),
     "hexa_esmm_gelu_bwd_ess": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
@@ -85,7 +86,7 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.hexa_abi_version() != 6:
+    if lib.hexa_abi_version() != 7:
         raise RuntimeError("hexa_moe: libhexa_moe_hip.so has an unexpected ABI version")
     _lib = lib
     return lib

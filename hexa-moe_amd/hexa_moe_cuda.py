@@ -66,17 +66,41 @@ def TOKEN_ASSIGN(token_idx_list, expert_idx_list, expanded_tokens_per_expert, ro
     _lib.check(rc, "TOKEN_ASSIGN")
 
 
+_route_cache = {}          # (list pointers, versions, sizes) -> Route; a handful of entries (one per live routing)
+_ROUTE_CACHE_MAX = 16
+
+
 def _route(token_idx_list, expert_idx_list, num_expanded_tokens, num_tokens, top_k, num_routings):
+    """Routing metadata of the operators for the caller's lists.  The reference's layer calls the matmul ops several
+    times per step with the same lists (impls/layers.py:256-274, 409-451); the metadata (and the ESTMM work plan
+    that hangs off it) is built once per list contents: the cache key holds the tensors' addresses and version
+    counters, so lists that were rewritten in place are rebuilt."""
     _i32(token_idx_list, "token_idx_list"); _i32(expert_idx_list, "expert_idx_list")
     if token_idx_list.numel() != expert_idx_list.numel():
         raise ValueError("token_idx_list and expert_idx_list differ in length")
+    key = (token_idx_list.data_ptr(), token_idx_list._version, expert_idx_list.data_ptr(), expert_idx_list._version,
+           token_idx_list.numel(), int(num_tokens), int(top_k), int(num_routings),
+           None if num_expanded_tokens is None else (num_expanded_tokens.data_ptr(), num_expanded_tokens._version))
+    hit = _route_cache.get(key)
+    if hit is not None:
+        return hit[0]
     if token_idx_list.numel() == num_tokens * top_k:     # exact lists: nothing to drop
-        return ops.route_from_lists(token_idx_list, expert_idx_list, int(num_tokens), int(top_k), int(num_routings))
-    if token_idx_list.numel() < num_tokens * top_k:
+        route = ops.route_from_lists(token_idx_list, expert_idx_list, int(num_tokens), int(top_k), int(num_routings))
+    elif token_idx_list.numel() < num_tokens * top_k:
         raise ValueError("the lists hold fewer than top_k * num_tokens entries")
-    _i32(num_expanded_tokens, "num_expanded_tokens")
-    return ops.route_from_padded_lists(token_idx_list, expert_idx_list, num_expanded_tokens, int(num_tokens),
-                                       int(top_k), int(num_routings))
+    else:
+        _i32(num_expanded_tokens, "num_expanded_tokens")
+        route = ops.route_from_padded_lists(token_idx_list, expert_idx_list, num_expanded_tokens, int(num_tokens),
+                                            int(top_k), int(num_routings))
+    if len(_route_cache) >= _ROUTE_CACHE_MAX:
+        _route_cache.pop(next(iter(_route_cache)))
+    # the entry keeps the list tensors alive, so their addresses cannot be reused by other lists while it exists
+    _route_cache[key] = (route, token_idx_list, expert_idx_list, num_expanded_tokens)
+    return route
+
+
+def clear_route_cache():
+    _route_cache.clear()
 
 
 def _check_flag(t, full, what):
@@ -107,11 +131,26 @@ def _fused(j_b, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, num_expand
         if not t.is_contiguous():
             raise TypeError("FUSED_GRAD: tensors must be contiguous")
     ws = torch.empty((k - 1) * T * int(num_in_dims), dtype=j_x.dtype, device=j_x.device) if (m2s and k > 1) else None
+    # balanced ESTMM and split ESS walk, as the layer's own calls get them (ops.estmm / ops.ess)
+    plan = scratch = ess_ws = None
+    slots = 0
+    mn = int(num_out_dims) * int(num_in_dims)
+    if j_y.dtype != torch.float32 and T * k >= 128 * E and mn % 4 == 0:
+        slots = min(2 * E, (256 << 20) // (mn * 4))
+        if slots >= 2:
+            plan = route.estmm_plan(slots)
+            scratch = torch.empty(slots * mn, dtype=torch.float32, device=j_y.device)
+        else:
+            slots = 0
+    if j_b is not None and T * k >= 256 * E:
+        ess_ws = torch.empty(8 * E * int(num_out_dims), dtype=torch.float32, device=j_y.device)
     rc = _lib.load().hexa_fused_grad(
         j_b.data_ptr() if j_b is not None else None, j_x.data_ptr(), j_w.data_ptr(), j_y.data_ptr(), w.data_ptr(),
         x.data_ptr(), route.blob.data_ptr(), int(bool(m2s)), 1, T, k, int(num_in_dims), int(num_out_dims), E,
         ops._dt(j_y), ops._dt(w), ops._dt(j_x), ops._dt(j_w), ops._dt(j_b) if j_b is not None else 0,
-        ws.data_ptr() if ws is not None else None, ops._stream())
+        ws.data_ptr() if ws is not None else None, plan.data_ptr() if plan is not None else None, slots,
+        scratch.data_ptr() if scratch is not None else None, ess_ws.data_ptr() if ess_ws is not None else None,
+        ess_ws.numel() if ess_ws is not None else 0, ops._stream())
     _lib.check(rc, "FUSED_GRAD")
 
 

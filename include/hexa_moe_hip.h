@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define HEXA_ABI_VERSION 6
+#define HEXA_ABI_VERSION 7
 
 /* element types */
 #define HEXA_F32 0
@@ -187,12 +187,17 @@ int hexa_ess_noalloc(void* db, const void* dy, const int32_t* route, int dy_per_
  *   m2s != 0: j_y [k,T,out], x [T,in] shared, j_x [T,in] (fc1 call, impls/layers.py:435-451)
  * act_dt: element type of j_y and x; w_dt: of w; jx_dt / jw_dt / jb_dt: of the results.
  * slot_ws: scratch of hexa_esmm for the m2s != 0 case ((top_k-1)*T*in elements of jx_dt) or NULL.
+ * plan / max_slots / estmm_scratch: as for hexa_estmm (a plan from hexa_estmm_plan for the same routing; NULL / 0 /
+ * NULL walks every expert's list in one workgroup).  ess_ws / ess_ws_floats: as for hexa_ess (NULL / 0: one pass).
+ * With them a caller of the fused op gets the balanced ESTMM and the split ESS walk; results do not depend on it
+ * beyond the order of the partial sums, which is fixed either way.
  * Replaces FUSED_GRAD / FUSED_GRAD_NO_BIAS (torch/hexa_moe_ops.cpp:119-275) ->
  * launch_fused_grad_{bias,no_bias}_{full,mix,half} (include/hexa_moe.h:74-181). */
 int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y, const void* w, const void* x,
                     const int32_t* route, int m2s, int accumulate, int num_tokens, int top_k, int in_dim,
                     int out_dim, int num_experts, int act_dt, int w_dt, int jx_dt, int jw_dt, int jb_dt,
-                    void* slot_ws, void* stream);
+                    void* slot_ws, const int32_t* plan, int max_slots, float* estmm_scratch, float* ess_ws,
+                    int64_t ess_ws_floats, void* stream);
 
 /* Steps 6-8 of the backward in one call: out[s][t][:] = (x[t][:] . w[e_s(t)]) * gelu'(y1[s][t][:]) (out, y1
  * [k,T,out_dim] in x's type; no bias) and db[e][:] (+)= the sum of expert e's rows of `out` (ESS of the result).

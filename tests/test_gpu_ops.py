@@ -125,7 +125,7 @@ def test_fused_grad(dev, dtype, m2s, T, d_in, d_out, E, k, skew):
     rc = _lib.load().hexa_fused_grad(jb.data_ptr(), jx.data_ptr(), jw.data_ptr(), jy_d.data_ptr(),
                                      w_d.data_ptr(), x_d.data_ptr(), route.blob.data_ptr(), int(m2s), 1,
                                      T, k, d_in, d_out, E, ops._dt(jy), ops._dt(w), 0, 0, 0, None,
-                                     torch.cuda.current_stream().cuda_stream)
+                                     None, 0, None, None, 0, torch.cuda.current_stream().cuda_stream)
     _lib.check(rc, "hexa_fused_grad")
     torch.cuda.synchronize()
     tol = TOL[dtype]
@@ -269,6 +269,7 @@ def test_reference_style_ops(dev, pad):
 
 def _reference_style_ops(dev, pad):
     import hexa_moe_cuda
+    hexa_moe_cuda.clear_route_cache()
     T, d_in, d_out, E, k = 600, 64, 128, 8, 2
     routing = make_routing(T, E, k, seed=21).to(torch.int32)
     x, W, b = make_linear(T, d_in, d_out, E, k, seed=22, dtype=F32, m2s=False)
@@ -310,6 +311,25 @@ def _reference_style_ops(dev, pad):
     torch.cuda.synchronize()
     assert_close(jb, jb_ref, 1e-5, "j_b"); assert_close(jx, jx_ref, 1e-5, "j_x"); assert_close(jw, jw_ref, 1e-5, "j_w")
     assert torch.equal(jx, jx2) and torch.equal(jw, jw2)
+    # the three matmul ops shared ONE build of the routing metadata (keyed on the list tensors); 16-bit operands
+    # with lists this long also take the balanced ESTMM (a plan made once per routing) and the split ESS walk
+    assert len(hexa_moe_cuda._route_cache) == 1
+    jb16 = torch.zeros(E, d_out, device=dev); jx16 = torch.zeros(T, d_in, device=dev, dtype=BF16)
+    jw16 = torch.zeros(E, d_out, d_in, device=dev)
+    hexa_moe_cuda.FUSED_GRAD(jb16.reshape(-1), jx16.reshape(-1), jw16.reshape(-1), jy.to(dev).to(BF16).reshape(-1),
+                             w.to(dev).to(BF16).reshape(-1), x.to(dev).to(BF16).reshape(-1), tok, exp, cum, False, False,
+                             True, T, k, d_in, d_out, E)
+    torch.cuda.synchronize()
+    assert len(hexa_moe_cuda._route_cache) == 1
+    assert_close(jb16, jb_ref, 2e-2, "j_b bf16"); assert_close(jx16, jx_ref, 2e-2, "j_x bf16"); assert_close(jw16, jw_ref, 2e-2, "j_w bf16")
+    # lists rewritten in place (same storage, new version) are not served from the cache
+    tok.add_(0)
+    jx3 = torch.zeros(T, d_in, device=dev); jw3 = torch.zeros(E, d_out, d_in, device=dev)
+    hexa_moe_cuda.FUSED_GRAD_NO_BIAS(jx3.reshape(-1), jw3.reshape(-1), jy.to(dev).reshape(-1), w.to(dev).reshape(-1),
+                                     x.to(dev).reshape(-1), tok, exp, cum, True, True, True, T, k, d_in, d_out, E)
+    torch.cuda.synchronize()
+    assert len(hexa_moe_cuda._route_cache) == 2 and torch.equal(jx3, jx2)
+    hexa_moe_cuda.clear_route_cache()
 
 
 def test_cpu_tensors_are_rejected(dev):

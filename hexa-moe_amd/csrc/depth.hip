@@ -153,6 +153,17 @@ extern "C" int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* 
                                                     w.router, stream));
     }
     RUN(hexa_route_build(idx, 0, k, 1, T, k, E, route, stream));
+    if (option(OPT_FFN_FUSED) == 1 && dma_path_enabled() &&
+        ffn16_fused_supported(T, k, d->d_in, d->hidden, d->d_out, d->act_dt, d->w_dt, d->b1_dt, d->b2_dt)) {
+        // fc1, GELU and fc2 in one kernel: event pair 0 brackets it (and the slot sum), pair 1 stays empty
+        RUN(ev.begin(0));
+        RUN(launch_ffn16_fused(y1, y2, y, x, fc1_w, fc1_b, fc2_w, fc2_b, route_view(route, T, k, E), d->d_in, d->hidden,
+                               d->d_out, d->act_dt, d->b1_dt, d->b2_dt, w.slot_ws, (hipStream_t)stream));
+        RUN(ev.end(0));
+        RUN(ev.begin(1));
+        RUN(ev.end(1));
+        return HEXA_OK;
+    }
     RUN(ev.begin(0));
     RUN(hexa_esmm(y1, x, fc1_w, fc1_b, route, 0, HEXA_W_OUT_IN, 0, T, k, d->d_in, d->hidden, E, d->act_dt, d->w_dt,
                   d->b1_dt, d->act_dt, HEXA_ACT_GELU, y2, nullptr, stream));

@@ -94,6 +94,7 @@ enum Opt {
     OPT_ESTMM_GROUP,    // HEXA_ESTMM_GROUP: row tiles per XCD run
     OPT_ESMM_STREAM,    // HEXA_ESMM_STREAM: 1 = results stored with the streaming hint
     OPT_ROUTE_KERNELS,  // HEXA_ROUTE_KERNELS: 3 = always the three-launch routing pass, 1 = one launch up to 65536 tokens
+    OPT_FFN_FUSED,      // HEXA_MOE_FFN_FUSED: 1 = hexa_moe_depth_forward runs fc1, GELU and fc2 in one kernel where it is covered
     OPT_COUNT
 };
 int option(int id);
@@ -102,6 +103,10 @@ bool esmm16_dma_supported(const EsmmArgs& a);
 bool esmm16_dma_colsum_supported(const EsmmArgs& a);
 bool esmm16_pipe_supported(const EsmmArgs& a);
 int launch_esmm16_pipe(const EsmmArgs& a, hipStream_t st);
+bool ffn16_fused_supported(int T, int k, int d_in, int hidden, int d_out, int act_dt, int w_dt, int b1_dt, int b2_dt);
+int launch_ffn16_fused(void* y1, void* y2, void* y, const void* x, const void* w1, const void* b1, const void* w2,
+                       const void* b2, const RouteView& r, int d_in, int hidden, int d_out, int act_dt, int b1_dt,
+                       int b2_dt, void* slot_ws, hipStream_t st);
 int launch_colsum_fold(const EsmmArgs& a, int mt_ub, int tile_rows, int ntn, int bn, hipStream_t st);
 int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, hipStream_t st);
 int launch_esmm16_dma(const EsmmArgs& a, hipStream_t s);

@@ -268,3 +268,40 @@ def test_depth_call_equals_operator_by_operator(dev, dtype, k, bias, loss):
     for u, v in zip(ga, gb):
         assert torch.equal(u, v)
     assert_close(dxa, dxb, 1e-6 if dtype == torch.float32 else 1e-2, "dx")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,d,E,k,bias", [(2500, 256, 16, 2, True), (2300, 384, 8, 1, True), (1900, 128, 5, 3, False),
+                                          (130, 512, 4, 2, True), (64, 128, 3, 1, True)])
+def test_one_kernel_ffn_forward(dev, dtype, T, d, E, k, bias):
+    """The depth call with fc1, GELU and fc2 in one kernel (library option "ffn_fused"): y against the oracle from
+    the module's own routing, and y, dx and every parameter gradient (which go through the y1 / y2 the kernel
+    saved) against the two-launch form."""
+    from hexa_moe import _lib
+    lib = _lib.load()
+    m = _module([d], [0], E=E, k=k, bias=bias, act=F.gelu, noise=1.0).to(dev).to(dtype).eval()
+    m.gates[0].wg.weight.data = m.gates[0].wg.weight.data.float()
+    g = torch.Generator().manual_seed(23)
+    x = torch.randn(T, d, generator=g).to(dtype).to(dev)
+    dy = torch.randn(T, d, generator=g).to(dtype).to(dev)
+    res = []
+    try:
+        for fused in (1, 0):
+            _lib.check(lib.hexa_set_option(b"ffn_fused", fused), "hexa_set_option")
+            m.zero_grad(set_to_none=True)
+            xi = x.clone().requires_grad_(True)
+            y, l_aux = m(0, xi)
+            torch.autograd.backward([y, l_aux], [dy, torch.full((), 2.0, device=dev)])
+            torch.cuda.synchronize()
+            params = [m.batched_fc1_w[0], m.batched_fc2_w[0]] + ([m.batched_fc1_bias[0], m.batched_fc2_bias[0]] if bias else [])
+            res.append((m.dispatch_params.routing_.clone().long().cpu(), y.detach().clone(), xi.grad.clone(), [p.grad.clone() for p in params]))
+    finally:
+        _lib.check(lib.hexa_set_option(b"ffn_fused", 0), "hexa_set_option")
+    (ra, ya, dxa, ga), (rb, yb, dxb, gb) = res
+    assert torch.equal(ra, rb)
+    y_ref, _ = _oracle_depth(m, 0, x.float().cpu(), ra, dy.float().cpu(), F.gelu, torch.float32)
+    assert_close(ya, y_ref, TOL[dtype], "y (one kernel) vs oracle")
+    assert_close(ya, yb, TOL[dtype] / 4, "y (one kernel) vs two launches")
+    assert_close(dxa, dxb, TOL[dtype] / 4, "dx")
+    for u, v in zip(ga, gb):
+        assert_close(u, v, TOL[dtype] / 4, "parameter gradient")

@@ -1,10 +1,11 @@
 // The gate's linear layer in fp32 on the matrix cores (v_mfma_f32_32x32x2_f32: fp32 multiply, fp32
 // accumulate), forward and backward, for token tensors of any supported type:
 //   logits[t][e] = sum_c x[t][c] * wg[e][c]                 (gate_fwd_kernel)
-//   dx[t][c]     = sum_e dlogits[t][e] * wg[e][c]           (gate_dx_kernel)
-//   dwg[e][c]    = sum_t dlogits[t][e] * x[t][c]            (gate_dwg_kernel + gate_dwg_reduce_kernel)
-// These are skinny products (E is a few dozen), HBM-bound on the token tensor; operands go from
-// global memory straight to registers.  The MFMA takes ONE contraction index per lane (lane l: row or
+//   dx[t][c]     = sum_e dlogits[t][e] * wg[e][c]           (gate_bwd_kernel, dx tasks)
+//   dwg[e][c]    = sum_t dlogits[t][e] * x[t][c]            (gate_bwd_kernel, dwg tasks + gate_dwg_reduce_kernel)
+// These are skinny products (E is a few dozen): little memory traffic, and at 64 cycles per fp32 MFMA the matrix
+// pipelines are what bounds them -- at 18432 tokens, d = 384 and 32 experts each product is 110592 MFMAs, 3.3 us
+// of the whole chip.  Operands go from global memory straight to registers.  The MFMA takes ONE contraction index per lane (lane l: row or
 // column l%32, index l/32), and which two indices one MFMA pairs is free as long as both operands
 // agree -- so a lane loads 8 (or 16) consecutive contraction indices in one go and feeds them to
 // consecutive MFMAs.  Where the fast output dimension is the token/gate row (dx, dwg), lane n owns 4
@@ -20,8 +21,9 @@ namespace {
 
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
-constexpr int GT = 32;          // tokens per workgroup (forward, dx)
-constexpr int DWG_TB = 64;      // tokens per workgroup (dwg)
+constexpr int GT = 32;          // tokens per workgroup (forward)
+constexpr int FWD_NB = 6;       // chunks of 8 contraction indices a wavefront of the forward kernel loads per trip
+constexpr int BWD_TB = 64;      // tokens per chunk of the backward tasks (and per dwg partial sum)
 
 __device__ __forceinline__ f32x16 zero16() {
     f32x16 z;
@@ -107,14 +109,21 @@ __global__ __launch_bounds__(256) void gate_fwd_kernel(float* __restrict__ logit
         const bool exp_ok = e0 + r < E;
         const float* wrow = wg + (size_t)(e0 + r) * d;
         f32x16 acc = zero16();
-        for (int c = c0; c < c1; ++c) {
-            const int piece = 2 * c + h;
-            const bool ok = piece < pieces;
-            float xv[8], wv[8];
-            LoadN<T, 8>::run(xrow + piece * 8, ok && tok_ok, xv);
-            LoadN<float, 8>::run(wrow + piece * 8, ok && exp_ok, wv);
+        // FWD_NB chunks per trip, every load of the trip issued before the first product: one memory latency per
+        // trip instead of one per chunk (a wavefront's share of d = 384 is 6 chunks = one trip)
+        for (int c = c0; c < c1; c += FWD_NB) {
+            float xv[FWD_NB][8], wv[FWD_NB][8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[i], wv[i], acc, 0, 0, 0);
+            for (int u = 0; u < FWD_NB; ++u) {
+                const int piece = 2 * (c + u) + h;
+                const bool ok = c + u < c1 && piece < pieces;
+                LoadN<T, 8>::run(xrow + (ok ? piece : 0) * 8, ok && tok_ok, xv[u]);
+                LoadN<float, 8>::run(wrow + (ok ? piece : 0) * 8, ok && exp_ok, wv[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < FWD_NB; ++u)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[u][i], wv[u][i], acc, 0, 0, 0);
         }
         __syncthreads();   // the previous expert block's partial sums have been consumed
 #pragma unroll
@@ -131,44 +140,60 @@ __global__ __launch_bounds__(256) void gate_fwd_kernel(float* __restrict__ logit
     }
 }
 
-// ---- dx: 32 tokens per workgroup, 128-column groups of the model dimension over the wavefronts ------
+// ---- backward: one task per WAVEFRONT ---------------------------------------------------------------------
+// The fp32 MFMA is slow (64 cycles for 32x32x2), the products are small, and a launch is over when its busiest
+// SIMD is: what matters is that every SIMD of the chip gets the same number of MFMAs.  So the work is cut into
+// tasks of equal length -- 128 MFMAs at 32 experts -- one per wavefront, four wavefronts (one per SIMD of a CU)
+// to a workgroup, nothing shared between them:
+//   dx task  (chunk, g): dx[64 tokens of the chunk][columns 128g .. 128g+127], two 32-token blocks one after the
+//                        other with the wavefront's slice of wg kept in registers (re-read per block above 32
+//                        experts)
+//   dwg task (chunk, eb, g): partial dwg[experts 32eb .. 32eb+31][columns 128g ..] over the chunk's 64 tokens
+// (with workgroups of three busy wavefronts and a fourth idle, and twice as many half-length dx tasks, the same
+// kernel took 28 us instead of 17 at 18432 tokens, d = 384, 32 experts: the MFMAs alone are 6.6 us of the chip).
 template <typename T>
-__device__ __forceinline__ void gate_dx_body(int block, T* __restrict__ dx, const float* __restrict__ dl,
+__device__ __forceinline__ void gate_dx_task(int chunk, int g, T* __restrict__ dx, const float* __restrict__ dl,
                                              const float* __restrict__ wg, int num_tokens, int d, int E) {
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = threadIdx.x & 63;
     const int r = lane & 31, h = lane >> 5;
-    const int t0 = block * GT;
-    const bool tok_ok = t0 + r < num_tokens;
-    const float* drow = dl + (size_t)(t0 + r) * E;
-    for (int g = wave; g * 128 < d; g += 4) {
-        const int col = g * 128 + 4 * r;
-        const bool col_ok = col < d;
+    const bool single = E <= 32;               // one pass over the experts: the wg slice is loaded once
+    const int col = g * 128 + 4 * r;
+    const bool col_ok = col < d;
+    float b[16][4];
+    auto load_b = [&](int e0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int e = e0 + 16 * h + i;
+            LoadN<float, 4>::run(wg + (size_t)(e < E ? e : 0) * d + (col_ok ? col : 0), col_ok && e < E, b[i]);
+        }
+    };
+    if (single) load_b(0);
+    for (int tb = 0; tb < BWD_TB / 32; ++tb) {
+        const int t0 = chunk * BWD_TB + tb * 32;
+        if (t0 >= num_tokens) break;
+        const bool tok_ok = t0 + r < num_tokens;
+        const float* drow = dl + (size_t)(tok_ok ? t0 + r : 0) * E;
         f32x16 acc[4] = {zero16(), zero16(), zero16(), zero16()};
         for (int e0 = 0; e0 < E; e0 += 32) {
             // this lane's contraction indices: experts e0 + 16h + 0..15
-            float a[16], b[16][4];
+            float a[16];
             if ((E & 3) == 0) {   // rows are 16-byte aligned: four float4 loads
 #pragma unroll
                 for (int i = 0; i < 16; i += 4) {
                     const int e = e0 + 16 * h + i;
                     float v[4];
-                    LoadN<float, 4>::run(drow + e, tok_ok && e < E, v);
+                    LoadN<float, 4>::run(drow + (e < E ? e : 0), tok_ok && e < E, v);
                     a[i] = v[0]; a[i + 1] = v[1]; a[i + 2] = v[2]; a[i + 3] = v[3];
                 }
             } else {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int e = e0 + 16 * h + i;
-                    a[i] = load1(drow + e, tok_ok && e < E);
+                    a[i] = load1(drow + (e < E ? e : 0), tok_ok && e < E);
                 }
             }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int e = e0 + 16 * h + i;
-                LoadN<float, 4>::run(wg + (size_t)e * d + col, col_ok && e < E, b[i]);
-            }
-            arrive(b);
+            if (!single) load_b(e0);
+            if (!single || tb == 0) arrive(b);
 #pragma unroll
             for (int i = 0; i < 16; ++i)
 #pragma unroll
@@ -184,73 +209,70 @@ __device__ __forceinline__ void gate_dx_body(int block, T* __restrict__ dx, cons
     }
 }
 
-// ---- dwg: partial sums over DWG_TB tokens per workgroup, then a reduction in workgroup order ---------
 template <typename T>
-__device__ __forceinline__ void gate_dwg_body(int part_idx, int e_block, float* __restrict__ part,
+__device__ __forceinline__ void gate_dwg_task(int chunk, int e_block, int g, float* __restrict__ part,
                                               const float* __restrict__ dl, const T* __restrict__ x, int num_tokens,
                                               int d, int E) {
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = threadIdx.x & 63;
     const int r = lane & 31, h = lane >> 5;
-    const int t0 = part_idx * DWG_TB;
+    const int t0 = chunk * BWD_TB;
     const int e0 = e_block * 32;
     const bool exp_ok = e0 + r < E;
-    float* out = part + (size_t)part_idx * E * d;
-    for (int g = wave; g * 128 < d; g += 4) {
-        const int col = g * 128 + 4 * r;
-        const bool col_ok = col < d;
-        f32x16 acc[4] = {zero16(), zero16(), zero16(), zero16()};
-        for (int i0 = 0; i0 < DWG_TB / 2; i0 += 8) {
-            float a[8], b[8][4];
+    float* out = part + (size_t)chunk * E * d;
+    constexpr int TRIPS = BWD_TB / 16;      // 8 MFMA steps (16 tokens) per trip
+    const int col = g * 128 + 4 * r;
+    const bool col_ok = col < d;
+    f32x16 acc[4] = {zero16(), zero16(), zero16(), zero16()};
+    // two trips of loads in flight: the next trip's loads are issued before this trip's products
+    float a[2][8], b[2][8][4];
+    auto load_trip = [&](int trip, float (&av)[8], float (&bv)[8][4]) {
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int t = t0 + 2 * (i0 + u) + h;          // this lane's contraction index: one token
-                const bool ok = t < num_tokens;
-                a[u] = load1(dl + (size_t)t * E + e0 + r, ok && exp_ok);
-                LoadN<T, 4>::run(x + (size_t)t * d + col, ok && col_ok, b[u]);
-            }
-            arrive(b);
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u][j], acc[j], 0, 0, 0);
+        for (int u = 0; u < 8; ++u) {
+            const int t = t0 + 2 * (8 * trip + u) + h;    // this lane's contraction index: one token
+            const bool ok = t < num_tokens;
+            av[u] = load1(dl + (size_t)(ok ? t : 0) * E + (exp_ok ? e0 + r : 0), ok && exp_ok);
+            LoadN<T, 4>::run(x + (size_t)(ok ? t : 0) * d + (col_ok ? col : 0), ok && col_ok, bv[u]);
         }
-        if (col_ok) {
+    };
+    load_trip(0, a[0], b[0]);
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int e = e0 + 8 * (v >> 2) + 4 * h + (v & 3);
-                if (e < E) store4<float>(out + (size_t)e * d + col, acc[0][v], acc[1][v], acc[2][v], acc[3][v]);
-            }
+    for (int trip = 0; trip < TRIPS; ++trip) {
+        if (trip + 1 < TRIPS) load_trip(trip + 1, a[(trip + 1) & 1], b[(trip + 1) & 1]);
+        arrive(b[trip & 1]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[trip & 1][u], b[trip & 1][u][j], acc[j], 0, 0, 0);
+    }
+    if (col_ok) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int e = e0 + 8 * (v >> 2) + 4 * h + (v & 3);
+            if (e < E) store4<float>(out + (size_t)e * d + col, acc[0][v], acc[1][v], acc[2][v], acc[3][v]);
         }
     }
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void gate_dx_kernel(T* __restrict__ dx, const float* __restrict__ dl,
-                                                      const float* __restrict__ wg, int num_tokens, int d, int E) {
-    gate_dx_body<T>(blockIdx.x, dx, dl, wg, num_tokens, d, E);
-}
-
-template <typename T>
-__global__ __launch_bounds__(256) void gate_dwg_kernel(float* __restrict__ part, const float* __restrict__ dl,
-                                                       const T* __restrict__ x, int num_tokens, int d, int E) {
-    gate_dwg_body<T>(blockIdx.x, blockIdx.y, part, dl, x, num_tokens, d, E);
-}
-
-// Both products in one launch: each of them alone leaves most of the chip waiting on memory latency, and they
-// share nothing but their inputs.  Workgroups alternate (two dx workgroups per dwg workgroup of the same 64
-// tokens, so the dlogits rows they both read are fetched once).
+// dx (when non-null) and the dwg partial sums (when `part` is non-null) in one launch: each product alone leaves
+// most of the chip waiting on memory latency, and they share nothing but their inputs.  Tasks are numbered chunk
+// by chunk -- the dx tasks of 64 tokens, then their dwg tasks -- so the dlogits rows both read are fetched once.
 template <typename T>
 __global__ __launch_bounds__(256) void gate_bwd_kernel(T* __restrict__ dx, float* __restrict__ part,
                                                        const float* __restrict__ dl, const T* __restrict__ x,
                                                        const float* __restrict__ wg, int num_tokens, int d, int E,
-                                                       int e_blocks) {
-    const int per = 2 + e_blocks;                 // workgroups per 64 tokens
-    const int grp = blockIdx.x / per, role = blockIdx.x - grp * per;
-    if (role < 2) {
-        if ((2 * grp + role) * GT < num_tokens) gate_dx_body<T>(2 * grp + role, dx, dl, wg, num_tokens, d, E);
+                                                       int ntasks) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int task = blockIdx.x * 4 + wave;
+    if (task >= ntasks) return;
+    const int groups = (d + 127) >> 7, e_blocks = (E + 31) >> 5;
+    const int n_dx = dx ? groups : 0, n_dwg = part ? groups * e_blocks : 0;
+    const int chunk = task / (n_dx + n_dwg), role = task - chunk * (n_dx + n_dwg);
+    if (role < n_dx) {
+        gate_dx_task<T>(chunk, role, dx, dl, wg, num_tokens, d, E);
     } else {
-        gate_dwg_body<T>(grp, role - 2, part, dl, x, num_tokens, d, E);
+        const int q = role - n_dx;
+        gate_dwg_task<T>(chunk, q / groups, q - (q / groups) * groups, part, dl, x, num_tokens, d, E);
     }
 }
 
@@ -283,24 +305,14 @@ __global__ __launch_bounds__(256) void gate_dwg_reduce_kernel(float* __restrict_
 template <typename T>
 int gate_backward_t(void* dx, float* dwg, const float* dl, const void* x, const float* wg, int T_, int d, int E, float* ws,
                     hipStream_t st) {
-    static_assert(DWG_TB == 2 * GT, "gate_bwd_kernel pairs two dx workgroups with one dwg workgroup");
-    if (dx && dwg) {
-        const int nparts = div_up(T_, DWG_TB), eb = div_up(E, 32);
-        hipLaunchKernelGGL(gate_bwd_kernel<T>, dim3(nparts * (2 + eb)), dim3(256), 0, st, (T*)dx, ws, dl, (const T*)x, wg,
-                           T_, d, E, eb);
-        HEXA_CHECK_LAUNCH("gate_bwd");
-    } else if (dx) {
-        hipLaunchKernelGGL(gate_dx_kernel<T>, dim3(div_up(T_, GT)), dim3(256), 0, st, (T*)dx, dl, wg, T_, d, E);
-        HEXA_CHECK_LAUNCH("gate_dx");
-    }
+    const int nchunks = div_up(T_, BWD_TB), groups = div_up(d, 128), eb = div_up(E, 32);
+    const int ntasks = nchunks * ((dx ? groups : 0) + (dwg ? groups * eb : 0));
+    hipLaunchKernelGGL(gate_bwd_kernel<T>, dim3(div_up(ntasks, 4)), dim3(256), 0, st, (T*)dx, dwg ? ws : nullptr, dl,
+                       (const T*)x, wg, T_, d, E, ntasks);
+    HEXA_CHECK_LAUNCH("gate_bwd");
     if (dwg) {
-        const int nparts = div_up(T_, DWG_TB);
-        if (!dx) {
-            hipLaunchKernelGGL(gate_dwg_kernel<T>, dim3(nparts, div_up(E, 32)), dim3(256), 0, st, ws, dl, (const T*)x, T_, d, E);
-            HEXA_CHECK_LAUNCH("gate_dwg");
-        }
         const long n4 = (long)E * d / 4;
-        hipLaunchKernelGGL(gate_dwg_reduce_kernel, dim3((unsigned)div_up(n4, 16)), dim3(256), 0, st, dwg, ws, nparts, n4);
+        hipLaunchKernelGGL(gate_dwg_reduce_kernel, dim3((unsigned)div_up(n4, 16)), dim3(256), 0, st, dwg, ws, nchunks, n4);
         HEXA_CHECK_LAUNCH("gate_dwg_reduce");
     }
     return HEXA_OK;
@@ -329,7 +341,7 @@ extern "C" int hexa_gate_logits(float* logits, const void* x, const float* wg, i
 
 extern "C" int hexa_gate_ws_floats(int T, int d, int E, int64_t* out) {
     if (!out || T < 0 || d < 1 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_gate_ws_floats: bad arguments");
-    *out = (int64_t)(T > 0 ? div_up(T, DWG_TB) : 1) * E * d;
+    *out = (int64_t)(T > 0 ? div_up(T, BWD_TB) : 1) * E * d;
     return HEXA_OK;
 }
 

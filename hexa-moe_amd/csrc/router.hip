@@ -18,8 +18,7 @@ constexpr int MAX_TOPK = 8;
 
 constexpr int ROUTER_TB = 64;   // tokens (= lanes) per workgroup of the softmax/top-k kernel
 
-constexpr int ROUTER_LDS_E = 240;   // up to this many experts the 64 x E tile is staged in LDS
-constexpr int ROUTER_P = ROUTER_TB + 1;   // pitch of one expert's 64 values
+constexpr int ROUTER_LDS_E = 240;   // up to this many experts the workgroup's 64 x E tile is staged in LDS
 
 // insertion of (cv, ci) into a descending list of k entries; strict '>' keeps the lower index on ties
 __device__ __forceinline__ void topk_insert(float (&best_v)[MAX_TOPK], int (&best_i)[MAX_TOPK], int k, float cv, int ci) {
@@ -32,52 +31,20 @@ __device__ __forceinline__ void topk_insert(float (&best_v)[MAX_TOPK], int (&bes
     }
 }
 
-// STAGED: the workgroup's 64 x E tile of (logits + noise) is brought into LDS with coalesced loads,
-// stored expert-major (conflict-free for one token per lane), turned into scores in place, summed per
-// expert and written back coalesced.  Otherwise every lane walks its own row in global memory (three
-// passes, L1-resident) and the per-expert sums are wavefront reductions.
-template <bool STAGED>
+// One token per lane for any number of experts: every lane walks its own row in global memory (three passes,
+// L1-resident) and the per-expert sums are wavefront reductions.  Used above ROUTER_LDS_E experts.
 __global__ __launch_bounds__(ROUTER_TB) void router_fwd_kernel(float* __restrict__ scores, int32_t* __restrict__ idx,
                                                          float* __restrict__ part_me, float* __restrict__ part_cnt,
                                                          const float* __restrict__ logits,
                                                          const float* __restrict__ noise, float noise_scale,
                                                          int num_tokens, int E, int k) {
-    extern __shared__ float sh[];          // me[E] column sums of the wavefront, cnt[E], then the tile
+    extern __shared__ float sh[];          // me[E] column sums of the wavefront, cnt[E]
     float* s_me = sh;
     float* s_cnt = sh + E;
-    float* tile = sh + 2 * E;              // [E][ROUTER_P]
     for (int i = threadIdx.x; i < 2 * E; i += blockDim.x) sh[i] = 0.f;
     const int lane = threadIdx.x;
-    const int t0 = blockIdx.x * ROUTER_TB;
-    const int t = t0 + lane;
+    const int t = blockIdx.x * ROUTER_TB + lane;
     const bool ok = t < num_tokens;
-    const int rows = min(ROUTER_TB, num_tokens - t0);
-    // staging geometry: lpr lanes (a power of two >= E, at most 64) per token row
-    int lpr = 1;
-    while (lpr < E && lpr < ROUTER_TB) lpr <<= 1;
-    const int rpi = ROUTER_TB / lpr, sub_r = lane / lpr, sub_e = lane & (lpr - 1);
-    if (STAGED) {
-        // 8 row groups per trip, loads first: the global latency is paid once per trip, not per row
-        for (int e0 = 0; e0 < E; e0 += lpr) {
-            const int e = e0 + sub_e;
-            for (int r0 = 0; r0 < rows; r0 += 8 * rpi) {
-                float v[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const int r = r0 + u * rpi + sub_r;
-                    const bool in = r < rows && e < E;
-                    const size_t g = (size_t)(t0 + r) * E + e;
-                    v[u] = in ? logits[g] : 0.f;
-                    if (in && noise) v[u] += noise_scale * noise[g];
-                }
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const int r = r0 + u * rpi + sub_r;
-                    if (r < rows && e < E) tile[e * ROUTER_P + r] = v[u];
-                }
-            }
-        }
-    }
     __syncthreads();
     // The selection is total: a row of NaN scores (NaN or +Inf logits) beats no entry, so the list starts out
     // as experts 0..k-1 and such a token stays routed (torch.topk also returns valid ids for NaN rows); its
@@ -86,54 +53,23 @@ __global__ __launch_bounds__(ROUTER_TB) void router_fwd_kernel(float* __restrict
     int best_i[MAX_TOPK];
 #pragma unroll
     for (int j = 0; j < MAX_TOPK; ++j) { best_v[j] = -INFINITY; best_i[j] = j; }
-    if (STAGED) {
-        float* col = tile + lane;          // this token's values, ROUTER_P apart
-        float mx = -INFINITY;
-        if (ok) {
-#pragma unroll 8
-            for (int e = 0; e < E; ++e) mx = fmaxf(mx, col[e * ROUTER_P]);
-            float sum = 0.f;
-#pragma unroll 8
-            for (int e = 0; e < E; ++e) {
-                const float ex = expf(col[e * ROUTER_P] - mx);
-                col[e * ROUTER_P] = ex;
-                sum += ex;
-            }
-            const float inv = 1.0f / sum;
-            float thresh = -INFINITY;      // k-th best so far
-#pragma unroll 4
-            for (int e = 0; e < E; ++e) {
-                const float sc = col[e * ROUTER_P] * inv;
-                col[e * ROUTER_P] = sc;
-                if (sc > thresh) {
-                    topk_insert(best_v, best_i, k, sc, e);
+    const float* lr = logits + (size_t)(ok ? t : 0) * E;
+    const float* nr = noise ? noise + (size_t)(ok ? t : 0) * E : nullptr;
+    float mx = -INFINITY;
+    for (int e = 0; e < E; ++e) mx = fmaxf(mx, nr ? lr[e] + noise_scale * nr[e] : lr[e]);
+    float sum = 0.f;
+    for (int e = 0; e < E; ++e) sum += expf((nr ? lr[e] + noise_scale * nr[e] : lr[e]) - mx);
+    const float inv = 1.0f / sum;
+    for (int e = 0; e < E; ++e) {        // uniform trip count: every lane takes part in the reductions
+        const float v = nr ? lr[e] + noise_scale * nr[e] : lr[e];
+        const float sc = ok ? expf(v - mx) * inv : 0.f;
+        if (ok) scores[(size_t)t * E + e] = sc;
+        topk_insert(best_v, best_i, k, sc, e);
+        // column sum over the wavefront: xor butterfly, a fixed summation tree
+        float r = sc;
 #pragma unroll
-                    for (int j = 0; j < MAX_TOPK; ++j)
-                        if (j == k - 1) thresh = best_v[j];
-                }
-            }
-        } else {
-            for (int e = 0; e < E; ++e) col[e * ROUTER_P] = 0.f;
-        }
-    } else {
-        const float* lr = logits + (size_t)(ok ? t : 0) * E;
-        const float* nr = noise ? noise + (size_t)(ok ? t : 0) * E : nullptr;
-        float mx = -INFINITY;
-        for (int e = 0; e < E; ++e) mx = fmaxf(mx, nr ? lr[e] + noise_scale * nr[e] : lr[e]);
-        float sum = 0.f;
-        for (int e = 0; e < E; ++e) sum += expf((nr ? lr[e] + noise_scale * nr[e] : lr[e]) - mx);
-        const float inv = 1.0f / sum;
-        for (int e = 0; e < E; ++e) {        // uniform trip count: every lane takes part in the reductions
-            const float v = nr ? lr[e] + noise_scale * nr[e] : lr[e];
-            const float sc = ok ? expf(v - mx) * inv : 0.f;
-            if (ok) scores[(size_t)t * E + e] = sc;
-            topk_insert(best_v, best_i, k, sc, e);
-            // column sum over the wavefront: xor butterfly, a fixed summation tree
-            float r = sc;
-#pragma unroll
-            for (int m = 32; m > 0; m >>= 1) r += __shfl_xor(r, m);
-            if (lane == 0) s_me[e] = r;
-        }
+        for (int m = 32; m > 0; m >>= 1) r += __shfl_xor(r, m);
+        if (lane == 0) s_me[e] = r;
     }
     if (ok) {
 #pragma unroll
@@ -142,27 +78,142 @@ __global__ __launch_bounds__(ROUTER_TB) void router_fwd_kernel(float* __restrict
         atomicAdd(&s_cnt[best_i[0]], 1.0f);            // exact: at most 64 ones per counter
     }
     __syncthreads();
-    if (STAGED) {
-        // per-expert sums over the 64 tokens, in token order; then the scores leave coalesced
-        for (int e = lane; e < E; e += ROUTER_TB) {
-            float m = 0.f;
-#pragma unroll 16
-            for (int r = 0; r < ROUTER_TB; ++r) m += tile[e * ROUTER_P + r];
-            s_me[e] = m;
-        }
-        for (int e0 = 0; e0 < E; e0 += lpr) {
-            const int e = e0 + sub_e;
-#pragma unroll 8
-            for (int r0 = 0; r0 < rows; r0 += rpi) {
-                const int r = r0 + sub_r;
-                if (r < rows && e < E) scores[(size_t)(t0 + r) * E + e] = tile[e * ROUTER_P + r];
-            }
-        }
-        __syncthreads();
-    }
     for (int e = threadIdx.x; e < E; e += blockDim.x) {
         part_me[(size_t)blockIdx.x * E + e] = s_me[e];
         part_cnt[(size_t)blockIdx.x * E + e] = s_cnt[e];
+    }
+}
+
+// Up to ROUTER_LDS_E experts: FOUR lanes per token (256 threads for the workgroup's 64 tokens).  One lane per
+// token leaves a 64-thread workgroup walking E-long dependent chains (max, exp and sum, selection) on a chip that
+// holds a few hundred such workgroups at once -- latency, not work, sets the time (18.8 us against 8.8 us at
+// 18432 tokens and 32 experts).  Lane q of a
+// token owns the experts e = q, q + 4, ...; maxima, sums and the top-k lists are combined over the four lanes
+// with quad shuffles.  The 64 x E tile sits token-major in LDS (pitch 4 x odd: the 64 lanes of a wavefront --
+// 16 tokens x 4 -- hit every bank twice, the minimum), is loaded and written back with coalesced 16-byte
+// accesses when E is a multiple of 4, and the per-expert sums run over it in token order.
+constexpr int ROUTER_G = 4;
+__host__ __device__ constexpr int router_pitch(int E) {
+    int p = (E + 3) / 4;            // in units of 4 floats
+    if ((p & 1) == 0) ++p;
+    return 4 * p;
+}
+
+__global__ __launch_bounds__(ROUTER_TB * ROUTER_G) void router_fwd4_kernel(
+    float* __restrict__ scores, int32_t* __restrict__ idx, float* __restrict__ part_me, float* __restrict__ part_cnt,
+    const float* __restrict__ logits, const float* __restrict__ noise, float noise_scale, int num_tokens, int E, int k) {
+    extern __shared__ float sh[];          // cnt[E], then the tile [64][P]
+    float* s_cnt = sh;
+    const int P = router_pitch(E);
+    float* tile = sh + ((E + 3) & ~3);
+    const int tid = threadIdx.x;
+    const int t0 = blockIdx.x * ROUTER_TB;
+    const int rows = min(ROUTER_TB, num_tokens - t0);
+    for (int i = tid; i < E; i += blockDim.x) s_cnt[i] = 0.f;
+    // ---- tile in: element i of the contiguous block [rows][E] ----
+    const size_t g0 = (size_t)t0 * E;
+    const int total = rows * E;
+    if ((E & 3) == 0) {
+        for (int i = tid * 4; i < total; i += blockDim.x * 4) {
+            float4 v = *reinterpret_cast<const float4*>(logits + g0 + i);
+            if (noise) {
+                const float4 n = *reinterpret_cast<const float4*>(noise + g0 + i);
+                v.x += noise_scale * n.x; v.y += noise_scale * n.y; v.z += noise_scale * n.z; v.w += noise_scale * n.w;
+            }
+            const int r = i / E, e = i - r * E;
+            *reinterpret_cast<float4*>(tile + r * P + e) = v;
+        }
+    } else {
+        for (int i = tid; i < total; i += blockDim.x) {
+            float v = logits[g0 + i];
+            if (noise) v += noise_scale * noise[g0 + i];
+            const int r = i / E, e = i - r * E;
+            tile[r * P + e] = v;
+        }
+    }
+    __syncthreads();
+    const int r = tid >> 2, q = tid & 3;
+    const int t = t0 + r;
+    const bool ok = r < rows;
+    float* row = tile + r * P;
+    // The selection is total: a row of NaN scores (NaN or +Inf logits) beats no entry, so the lists start out as
+    // the lanes' own experts in index order and such a token ends up with experts 0..k-1 (torch.topk also returns
+    // valid ids for NaN rows); its NaN then reaches the output through the token's own features and the loss
+    // through the score sums.
+    float bv[MAX_TOPK];
+    int bi[MAX_TOPK];
+#pragma unroll
+    for (int j = 0; j < MAX_TOPK; ++j) { bv[j] = -INFINITY; bi[j] = q + ROUTER_G * j; }
+    if (ok) {
+        float mx = -INFINITY;
+        for (int e = q; e < E; e += ROUTER_G) mx = fmaxf(mx, row[e]);
+        mx = fmaxf(mx, __shfl_xor(mx, 1));
+        mx = fmaxf(mx, __shfl_xor(mx, 2));
+        float sum = 0.f;
+        for (int e = q; e < E; e += ROUTER_G) {
+            const float ex = expf(row[e] - mx);
+            row[e] = ex;
+            sum += ex;
+        }
+        sum += __shfl_xor(sum, 1);         // (s0 + s1) + (s2 + s3) on every lane of the quad
+        sum += __shfl_xor(sum, 2);
+        const float inv = 1.0f / sum;
+        for (int e = q; e < E; e += ROUTER_G) {
+            const float sc = row[e] * inv;
+            row[e] = sc;
+            topk_insert(bv, bi, k, sc, e);  // ascending e, strict '>': the lower index stays ahead on ties
+        }
+    } else {
+        for (int e = q; e < E; e += ROUTER_G) row[e] = 0.f;
+    }
+    // merge the four lists: k rounds, each takes the best head (greater score; lower index on ties)
+    int pick[MAX_TOPK];
+#pragma unroll
+    for (int j = 0; j < MAX_TOPK; ++j) {
+        pick[j] = 0;
+        if (j < k) {
+            float hv = bv[0];
+            int hi = bi[0];
+#pragma unroll
+            for (int m = 1; m <= 2; m <<= 1) {
+                const float ov = __shfl_xor(hv, m);
+                const int oi = __shfl_xor(hi, m);
+                if (ov > hv || (ov == hv && oi < hi)) { hv = ov; hi = oi; }
+            }
+            pick[j] = hi;
+            if (hi == bi[0]) {
+#pragma unroll
+                for (int m = 0; m + 1 < MAX_TOPK; ++m) { bv[m] = bv[m + 1]; bi[m] = bi[m + 1]; }
+                bv[MAX_TOPK - 1] = -INFINITY;
+                bi[MAX_TOPK - 1] = 0x7fffffff;
+            }
+        }
+    }
+    if (ok) {
+#pragma unroll
+        for (int j = 0; j < MAX_TOPK; ++j)
+            if (j < k && (j & 3) == q) idx[(size_t)t * k + j] = pick[j];
+        if (q == 0) atomicAdd(&s_cnt[pick[0]], 1.0f);   // exact: at most 64 ones per counter
+    }
+    __syncthreads();
+    // per-expert sums over the 64 tokens, in token order; the scores leave coalesced
+    for (int e = tid; e < E; e += blockDim.x) {
+        float m = 0.f;
+#pragma unroll 16
+        for (int rr = 0; rr < ROUTER_TB; ++rr) m += tile[rr * P + e];
+        part_me[(size_t)blockIdx.x * E + e] = m;
+        part_cnt[(size_t)blockIdx.x * E + e] = s_cnt[e];
+    }
+    if ((E & 3) == 0) {
+        for (int i = tid * 4; i < total; i += blockDim.x * 4) {
+            const int rr = i / E, e = i - rr * E;
+            *reinterpret_cast<float4*>(scores + g0 + i) = *reinterpret_cast<const float4*>(tile + rr * P + e);
+        }
+    } else {
+        for (int i = tid; i < total; i += blockDim.x) {
+            const int rr = i / E, e = i - rr * E;
+            scores[g0 + i] = tile[rr * P + e];
+        }
     }
 }
 
@@ -450,10 +501,10 @@ extern "C" int hexa_router_forward(float* scores, int32_t* idx, float* me, float
     float* part_me = ws;
     float* part_cnt = ws + (size_t)nb * E;
     if (E <= ROUTER_LDS_E)
-        hipLaunchKernelGGL(router_fwd_kernel<true>, dim3(nb), dim3(ROUTER_TB), sizeof(float) * (2 * E + E * ROUTER_P), st,
-                           scores, idx, part_me, part_cnt, logits, noise, noise_scale, T, E, k);
+        hipLaunchKernelGGL(router_fwd4_kernel, dim3(nb), dim3(ROUTER_TB * ROUTER_G), sizeof(float) * (((E + 3) & ~3) + ROUTER_TB * router_pitch(E)),
+                           st, scores, idx, part_me, part_cnt, logits, noise, noise_scale, T, E, k);
     else
-        hipLaunchKernelGGL(router_fwd_kernel<false>, dim3(nb), dim3(ROUTER_TB), sizeof(float) * 2 * E, st, scores, idx,
+        hipLaunchKernelGGL(router_fwd_kernel, dim3(nb), dim3(ROUTER_TB), sizeof(float) * 2 * E, st, scores, idx,
                            part_me, part_cnt, logits, noise, noise_scale, T, E, k);
     HEXA_CHECK_LAUNCH("router_fwd");
     const int nch = E <= 256 ? 32 : (8192 / E > 0 ? 8192 / E : 1);

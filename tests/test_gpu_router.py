@@ -48,7 +48,8 @@ def test_gate_backward(dev, dtype, T, d, E):
     assert torch.equal(dwg, dwg2)
 
 
-@pytest.mark.parametrize("T,E,k", [(1000, 32, 2), (18432, 32, 2), (2048, 8, 1), (513, 70, 3), (64, 4, 4)])
+@pytest.mark.parametrize("T,E,k", [(1000, 32, 2), (18432, 32, 2), (2048, 8, 1), (513, 70, 3), (64, 4, 4), (257, 300, 2), (130, 9, 8),
+                                   (200, 240, 5)])
 @pytest.mark.parametrize("with_noise", [False, True])
 def test_router_forward_and_backward(dev, T, E, k, with_noise):
     from hexa_moe import ops

@@ -24,6 +24,7 @@ OptEntry g_opts[OPT_COUNT] = {
     {"general_kernels", "HEXA_MOE_GENERAL_KERNELS", 0, false}, {"esmm_map", "HEXA_ESMM_MAP", 0, false},
     {"esmm_group", "HEXA_ESMM_GROUP", 0, false},  {"estmm_group", "HEXA_ESTMM_GROUP", 0, false},
     {"esmm_stream", "HEXA_ESMM_STREAM", 0, false}, {"route_kernels", "HEXA_ROUTE_KERNELS", 0, false},
+    {"batch", "HEXA_MOE_BATCH", 0, false},
     {"ffn_fused", "HEXA_MOE_FFN_FUSED", 0, false},
 };
 }  // namespace

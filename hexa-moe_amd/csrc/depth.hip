@@ -7,7 +7,7 @@
 // FusedMoE_Shared_CudaCore.forward (impls/layers.py:99-277) and .backward (impls/layers.py:280-474).
 #include <algorithm>
 
-#include "hexa_internal.h"
+#include "small_tasks.h"
 
 namespace hexa {
 namespace {
@@ -37,7 +37,7 @@ int estmm_slots(const hexa_moe_depth_desc& d, int out_dim, int in_dim) {
     return slots >= 2 ? (int)slots : 0;
 }
 
-struct FwdWs { float* router; void* slot_ws; int64_t bytes; };
+struct FwdWs { float* router; int32_t* hist; void* slot_ws; int64_t bytes; };
 struct BwdWs {
     float* dlogits; float* gate; float* ess; float* colsum; int64_t colsum_floats; int32_t* plan; float* estmm;
     int slots; void* slot_ws; void* dx_gate; int64_t bytes;
@@ -48,6 +48,9 @@ int carve_forward(const hexa_moe_depth_desc& d, void* ws, FwdWs* out) {
     int64_t rf = 0;
     if (int rc = hexa_router_ws_floats(d.num_tokens, d.num_experts, &rf)) return rc;
     out->router = static_cast<float*>(c.take(rf * 4));
+    // the routing pass's histogram over the router's workgroups (64 tokens each), counted by the router itself
+    out->hist = static_cast<int32_t*>(c.take((int64_t)d.top_k * div_up(std::max(d.num_tokens, 1), router_tokens_per_workgroup()) *
+                                              d.num_experts * 4));
     out->slot_ws = d.top_k > 1 ? c.take((int64_t)(d.top_k - 1) * d.num_tokens * d.d_out * elem_size(d.act_dt)) : nullptr;
     out->bytes = c.used;
     return HEXA_OK;
@@ -130,8 +133,8 @@ extern "C" int hexa_moe_depth_ws_bytes(const hexa_moe_depth_desc* d, int64_t* fo
 extern "C" int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* x, const float* wg, const float* noise,
                                       const void* fc1_w, const void* fc1_b, const void* fc2_w, const void* fc2_b,
                                       float* logits, float* scores, int32_t* idx, float* thr, float* stats,
-                                      int32_t* route, void* y1, void* y2, void* y, void* ws, int64_t ws_bytes,
-                                      void* const* events, int num_events, void* stream) {
+                                      int32_t* route, int32_t* plan, void* y1, void* y2, void* y, void* ws,
+                                      int64_t ws_bytes, void* const* events, int num_events, void* stream) {
     const char* who = "hexa_moe_depth_forward";
     RUN(check_desc(who, d));
     if (!x || !fc1_w || !fc2_w || !idx || !route || !y1 || !y2 || !y || !ws) HEXA_FAIL(HEXA_ERR_ARG, "%s: null pointer", who);
@@ -141,18 +144,34 @@ extern "C" int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* 
     if (ws_bytes < w.bytes) HEXA_FAIL(HEXA_ERR_ARG, "%s: workspace of %lld bytes, %lld needed", who, (long long)ws_bytes, (long long)w.bytes);
     const int T = d->num_tokens, k = d->top_k, E = d->num_experts;
     const EventPairs ev{events, num_events, (hipStream_t)stream};
+    // the work plan of the backward's ESTMM calls depends on the routing only: made here when the caller keeps it
+    const int plan_slots = std::min(estmm_slots(*d, d->hidden, d->d_out), estmm_slots(*d, d->hidden, d->d_in));
+    if (plan && plan_slots < 2) plan = nullptr;
+    bool routed = false;
     if (wg) {
         if (!logits || !scores || !stats || (d->loss == 1 && !thr)) HEXA_FAIL(HEXA_ERR_ARG, "%s: null router state", who);
         RUN(hexa_gate_logits(logits, x, wg, T, d->d_in, E, d->act_dt, stream));
-        if (d->loss == 0)
+        if (d->loss == 0 && router_hist_supported(E)) {
+            // three launches for router, loss, routing pass and plan: the router counts its own tokens for the routing
+            // pass, whose scan launch carries the loss and whose scatter launch carries the plan
+            RUN(router_forward_check(T, E, k, true));
+            RUN(launch_router_fwd(scores, idx, logits, noise, d->noise_scale, T, E, k, w.router, w.hist, (hipStream_t)stream));
+            RUN(launch_route_from_hist(idx, T, k, E, route, w.hist, router_tokens_per_workgroup(), stats + 2 * E, stats,
+                                       stats + E, w.router, plan, plan_slots, (hipStream_t)stream));
+            routed = true;
+        } else if (d->loss == 0) {
             RUN(hexa_router_forward(scores, idx, stats, stats + E, stats + 2 * E, logits, noise, d->noise_scale, T, E, k,
                                     w.router, stream));
-        else
+        } else {
             RUN(hexa_router_forward_load_importance(scores, idx, thr, stats, stats + E, stats + 2 * E, stats + 3 * E,
                                                     stats + 4 * E, logits, noise, d->noise_scale, d->sigma, T, E, k,
                                                     w.router, stream));
+        }
     }
-    RUN(hexa_route_build(idx, 0, k, 1, T, k, E, route, stream));
+    if (!routed) {
+        RUN(hexa_route_build(idx, 0, k, 1, T, k, E, route, stream));
+        if (plan) RUN(hexa_estmm_plan(plan, route, T, k, E, plan_slots, stream));
+    }
     if (option(OPT_FFN_FUSED) == 1 && dma_path_enabled() &&
         ffn16_fused_supported(T, k, d->d_in, d->hidden, d->d_out, d->act_dt, d->w_dt, d->b1_dt, d->b2_dt)) {
         // fc1, GELU and fc2 in one kernel: event pair 0 brackets it (and the slot sum), pair 1 stays empty
@@ -178,9 +197,9 @@ extern "C" int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* 
 extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void* dy, const float* grad_l_aux,
                                        const void* x, const float* wg, const void* fc1_w, const void* fc2_w,
                                        const float* scores, const int32_t* idx, const float* thr, const float* stats,
-                                       const int32_t* route, const void* y1, const void* y2, void* dx, float* dwg,
-                                       void* dw1, void* db1, void* dw2, void* db2, void* dy1, void* ws,
-                                       int64_t ws_bytes, void* const* events, int num_events, void* stream) {
+                                       const int32_t* route, const int32_t* plan, const void* y1, const void* y2,
+                                       void* dx, float* dwg, void* dw1, void* db1, void* dw2, void* db2, void* dy1,
+                                       void* ws, int64_t ws_bytes, void* const* events, int num_events, void* stream) {
     const char* who = "hexa_moe_depth_backward";
     RUN(check_desc(who, d));
     if (!dy || !x || !fc1_w || !fc2_w || !route || !y1 || !y2 || !dy1 || !ws) HEXA_FAIL(HEXA_ERR_ARG, "%s: null pointer", who);
@@ -193,19 +212,55 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
     const bool gate_path = wg && grad_l_aux && (dx || dwg);
     if (gate_path && (!scores || !stats || (d->loss == 1 && (!thr || !idx)))) HEXA_FAIL(HEXA_ERR_ARG, "%s: null router state", who);
 
+    // The second-stage and elementwise kernels of this call are independent of most of what surrounds them, and a
+    // launch of its own costs each of them 5-7 us: where the element type has a batch kernel they are collected
+    // as tasks and run four launches (A-D) instead of nine, each placed where the stream order allows:
+    //   A  ESS(dy) partial sums, router backward              -- before anything that needs them
+    //   B  fix-up of dW2, fold of the ESS partial sums        -- behind ESTMM dW2 (the scratch is reused by dW1)
+    //   C  fix-up of dW1, fold of db1's column sums           -- behind ESTMM dW1
+    //   D  slot sum of dx (+ the gate's share), gate dwg fold -- behind the dx kernel
+    // A launcher that cannot put its task into the batch offered (other element type, general kernels) launches it
+    // on the spot, which is always in order.
+    const bool batching = batch_supported(d->act_dt) && option(OPT_BATCH) != 2;
+    SmallBatch A, B, C, D;
+    A.dt = B.dt = C.dt = D.dt = d->act_dt;
+    struct Guard { ~Guard() { defer_targets() = DeferTargets(); } } guard;
+    DeferTargets& tg = defer_targets();
+    hipStream_t st = (hipStream_t)stream;
+
     // step 4: db2 = ESS(dy)
-    if (db2) RUN(hexa_ess(db2, dy, route, 0, 0, T, k, d->d_out, E, d->act_dt, d->gb2_dt, w.ess, (int64_t)8 * E * d->d_out, stream));
+    if (db2) {
+        if (batching) { tg.ess = &A; tg.ess_fold = &B; }
+        RUN(hexa_ess(db2, dy, route, 0, 0, T, k, d->d_out, E, d->act_dt, d->gb2_dt, w.ess, (int64_t)8 * E * d->d_out, stream));
+        tg = DeferTargets();
+    }
+    // the gate path, part 1: d l_aux / d logits through the softmax (and the threshold)
+    if (gate_path) {
+        if (batching) tg.router_bwd = &A;
+        if (d->loss == 0)
+            RUN(hexa_router_backward(w.dlogits, scores, stats + E, grad_l_aux, T, E, stream));
+        else
+            RUN(hexa_router_backward_load_importance(w.dlogits, scores, thr, idx, stats + 2 * E, stats + 3 * E, grad_l_aux,
+                                                     d->sigma, T, E, k, stream));
+        tg = DeferTargets();
+    }
+    RUN(batch_flush(A, st));
     const bool planned = w.slots >= 2 && (dw1 || dw2);
-    if (planned) RUN(hexa_estmm_plan(w.plan, route, T, k, E, w.slots, stream));
+    if (planned && !plan) RUN(hexa_estmm_plan(w.plan, route, T, k, E, w.slots, stream));
+    if (planned && plan) w.plan = const_cast<int32_t*>(plan);   // made by the forward for the same routing and slot count
     // step 5: dW2 = ESTMM(act(y1), dy): the per-slot operand supplies the rows of dW2 [E][hidden][d_out]
     if (dw2) {
+        if (batching) tg.fixup = &B;
         RUN(ev.begin(2));
         RUN(hexa_estmm(dw2, y2, dy, route, 1, 0, 0, T, k, d->hidden, d->d_out, E, d->act_dt, d->gw2_dt,
                        planned ? w.plan : nullptr, planned ? w.slots : 0, planned ? w.estmm : nullptr, stream));
         RUN(ev.end(2));
+        tg = DeferTargets();
     }
+    RUN(batch_flush(B, st));
     if (dx || dw1 || db1) {
         // steps 6-8: dy1 = (dy . W2^T) * gelu'(y1), db1 = ESS(dy1)
+        if (batching) tg.colsum_fold = &C;
         RUN(ev.begin(0));
         if (db1)
             RUN(hexa_esmm_gelu_bwd_ess(dy1, db1, dy, fc2_w, y1, route, HEXA_W_OUT_IN, 0, T, k, d->d_out, d->hidden, E,
@@ -214,31 +269,33 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
             RUN(hexa_esmm(dy1, dy, fc2_w, nullptr, route, 0, HEXA_W_OUT_IN, 0, T, k, d->d_out, d->hidden, E, d->act_dt,
                           d->w_dt, HEXA_F32, d->act_dt, HEXA_ACT_GELU_BWD, const_cast<void*>(y1), nullptr, stream));
         RUN(ev.end(0));
+        tg = DeferTargets();
         // step 9: dW1 = ESTMM(dy1, x)
         if (dw1) {
+            if (batching) tg.fixup = &C;
             RUN(ev.begin(3));
             RUN(hexa_estmm(dw1, dy1, x, route, 1, 0, 0, T, k, d->hidden, d->d_in, E, d->act_dt, d->gw1_dt,
                            planned ? w.plan : nullptr, planned ? w.slots : 0, planned ? w.estmm : nullptr, stream));
             RUN(ev.end(3));
+            tg = DeferTargets();
         }
     }
-    // the gate path: d l_aux / d logits through the softmax (and the threshold), then through the projection
+    // the gate path, part 2: through the projection
     bool gate_dx_in_ws = false;
     if (gate_path) {
-        if (d->loss == 0)
-            RUN(hexa_router_backward(w.dlogits, scores, stats + E, grad_l_aux, T, E, stream));
-        else
-            RUN(hexa_router_backward_load_importance(w.dlogits, scores, thr, idx, stats + 2 * E, stats + 3 * E, grad_l_aux,
-                                                     d->sigma, T, E, k, stream));
         // With several slots on the 16-bit fast path the slot sum of step 10 adds the gate's share as one more
         // addend; otherwise the gate's share is written into dx first and step 10 accumulates onto it.
         gate_dx_in_ws = dx && k > 1 && d->act_dt != HEXA_F32 && d->w_dt == d->act_dt && dma_path_enabled() &&
                         (d->hidden % 32) == 0 && (d->d_in % 8) == 0;
+        if (batching) tg.dwg_reduce = &D;
         RUN(hexa_gate_backward(dx ? (gate_dx_in_ws ? w.dx_gate : dx) : nullptr, dwg, w.dlogits, x, wg, T, d->d_in, E,
                                d->act_dt, w.gate, stream));
+        tg = DeferTargets();
     }
+    RUN(batch_flush(C, st));
     // step 10: dx = ESMM(dy1, W1), summed over the slots (+ the gate's share)
     if (dx) {
+        if (batching) tg.sum_slots = &D;
         RUN(ev.begin(1));
         bool used = false;
         const int acc = gate_path && !gate_dx_in_ws ? 1 : 0;
@@ -247,6 +304,8 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
                       &used, stream));
         if (gate_dx_in_ws && !used) HEXA_FAIL(HEXA_ERR_LAUNCH, "%s: internal: the gate's input gradient was not added", who);
         RUN(ev.end(1));
+        tg = DeferTargets();
     }
+    RUN(batch_flush(D, st));
     return HEXA_OK;
 }

@@ -11,110 +11,15 @@
 // Replaces the ESS task of fused_grad_bias_kernel_vectorized_* (kernels/fused_ops_full.cu:372-431).
 #include <algorithm>
 
-#include "hexa_internal.h"
+#include "small_bodies.h"
 
 namespace hexa {
 namespace {
 
-template <typename T> struct Vec16;  // 16 bytes of T
-template <> struct Vec16<float> { static constexpr int N = 4; };
-template <> struct Vec16<__bf16> { static constexpr int N = 8; };
-template <> struct Vec16<_Float16> { static constexpr int N = 8; };
-
-struct EssK {
-    const void* dy; void* db;
-    const int32_t* token_ids; const int32_t* offsets;
-    int T, k, E, N, dy_slot_rows, accumulate, db_dt;
-    float* ws; int splits;   // splits > 1: workgroup z sums the z-th part of every segment into ws[z][E][N]
-};
-
 template <typename T>
-__global__ __launch_bounds__(256) void ess_kernel(EssK p) {
-    constexpr int V = Vec16<T>::N;
-    constexpr int STRIP = 8 * V;  // columns per workgroup
-    constexpr int U = 8;          // rows in flight per lane: 256 rows (32 KiB) per workgroup step
-    __shared__ float red[4][STRIP];
-    const int e = blockIdx.y;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int cl = lane & 7, rg = lane >> 3;
-    const int col = blockIdx.x * STRIP + cl * V;
-    const bool col_ok = col < p.N;
-    const T* dy = reinterpret_cast<const T*>(p.dy);
+__global__ __launch_bounds__(256) void ess_kernel(EssK p) { ess_body<T>(p, blockIdx.x); }
 
-    float acc[V];
-#pragma unroll
-    for (int i = 0; i < V; ++i) acc[i] = 0.f;
-
-    bool any = false;
-    for (int s = 0; s < p.k; ++s) {
-        int beg = p.offsets[(size_t)s * (p.E + 1) + e];
-        int end = p.offsets[(size_t)s * (p.E + 1) + e + 1];
-        any = any || end > beg;
-        if (p.splits > 1) {
-            const int part = (end - beg + p.splits - 1) / p.splits;
-            beg = min(end, beg + (int)blockIdx.z * part);
-            end = min(end, beg + part);
-        }
-        const int32_t* tok = p.token_ids + (size_t)s * p.T;
-        const T* base = dy + (size_t)p.dy_slot_rows * s * p.N + col;
-        // this lane's rows: beg + wave*8 + rg + 32*u + 256*step; the token ids of the next step are
-        // fetched while the rows of the current one are in flight
-        const int r_lane = beg + wave * 8 + rg;
-        int ids[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) { const int r = r_lane + 32 * u; ids[u] = r < end ? tok[r] : -1; }
-        for (int r0 = r_lane; r0 < end; r0 += 32 * U) {
-            union { uint4 u; T e[V]; } v[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-                v[u].u = (ids[u] >= 0 && col_ok) ? *reinterpret_cast<const uint4*>(base + (size_t)ids[u] * p.N)
-                                                 : make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-            for (int u = 0; u < U; ++u) { const int r = r0 + 32 * U + 32 * u; ids[u] = r < end ? tok[r] : -1; }
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-#pragma unroll
-                for (int i = 0; i < V; ++i) acc[i] += Cvt<T>::to_f(v[u].e[i]);
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < V; ++i) {
-        float a = acc[i];
-        a += __shfl_xor(a, 8);
-        a += __shfl_xor(a, 16);
-        a += __shfl_xor(a, 32);
-        acc[i] = a;
-    }
-    if (rg == 0) {
-#pragma unroll
-        for (int i = 0; i < V; ++i) red[wave][cl * V + i] = acc[i];
-    }
-    __syncthreads();
-    if (tid < STRIP) {
-        const int c = blockIdx.x * STRIP + tid;
-        const float v = red[0][tid] + red[1][tid] + red[2][tid] + red[3][tid];
-        if (p.splits > 1) {
-            if (c < p.N) p.ws[((size_t)blockIdx.z * p.E + e) * p.N + c] = v;
-        } else if (c < p.N && (any || !p.accumulate)) {
-            store_out(p.db, (size_t)e * p.N + c, v, p.db_dt, p.accumulate != 0);
-        }
-    }
-}
-
-// db (+)= ws[0] + ws[1] + ... in that order
-__global__ __launch_bounds__(256) void ess_fold_kernel(void* __restrict__ db, const float* __restrict__ ws, long n,
-                                                       int splits, int db_dt, int accumulate) {
-    const long i = (long)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    // all parts' loads in flight at once (at most 8 parts), added in part order
-    float part[8];
-#pragma unroll
-    for (int z = 0; z < 8; ++z) part[z] = ws[(size_t)min(z, splits - 1) * n + i];
-    float v = part[0];
-#pragma unroll
-    for (int z = 1; z < 8; ++z) v += z < splits ? part[z] : 0.f;
-    store_out(db, (size_t)i, v, db_dt, accumulate != 0);
-}
+__global__ __launch_bounds__(256) void ess_fold_kernel(EssFoldK p) { ess_fold_body(p, blockIdx.x); }
 
 template <typename T>
 int launch_ess_t(const EssArgs& a, hipStream_t st) {
@@ -135,13 +40,22 @@ int launch_ess_t(const EssArgs& a, hipStream_t st) {
     if (a.ws && per_part > 0 && avg_rows >= 256) splits = (int)std::min<long>(8, a.ws_floats / per_part);
     if (splits < 2) splits = 1;
     p.ws = a.ws; p.splits = splits;
-    dim3 grid(div_up(a.out_dim, STRIP), a.r.E, splits);
-    hipLaunchKernelGGL((ess_kernel<T>), grid, dim3(256), 0, st, p);
-    HEXA_CHECK_LAUNCH("ess");
+    p.gx = div_up(a.out_dim, STRIP); p.gy = a.r.E;
+    SmallTask t;
+    t.kind = TASK_ESS; t.ess = p; t.blocks = p.gx * p.gy * splits;
+    if (t.blocks == 0) return HEXA_OK;
+    if (!defer_task(defer_targets().ess, t, a.dy_dt)) {
+        hipLaunchKernelGGL((ess_kernel<T>), dim3(t.blocks), dim3(256), 0, st, p);
+        HEXA_CHECK_LAUNCH("ess");
+    }
     if (splits > 1) {
-        hipLaunchKernelGGL(ess_fold_kernel, dim3((unsigned)((per_part + 255) / 256)), dim3(256), 0, st, a.db, a.ws, per_part,
-                           splits, a.db_dt, a.accumulate);
-        HEXA_CHECK_LAUNCH("ess_fold");
+        SmallTask f;
+        f.kind = TASK_ESS_FOLD; f.ess_fold = EssFoldK{a.db, a.ws, per_part, splits, a.db_dt, a.accumulate};
+        f.blocks = (int)((per_part + 255) / 256);
+        if (!defer_task(defer_targets().ess_fold, f)) {
+            hipLaunchKernelGGL(ess_fold_kernel, dim3(f.blocks), dim3(256), 0, st, f.ess_fold);
+            HEXA_CHECK_LAUNCH("ess_fold");
+        }
     }
     return HEXA_OK;
 }
@@ -187,55 +101,30 @@ int launch_gelu_bwd_t(void* dy1, const void* dy2, const void* y1, int64_t n, hip
     return HEXA_OK;
 }
 
-// out[i] += ws[0][i] + ws[1][i] + ... in fp32, slot order (the deterministic reduction behind the
-// one-launch slot sum of ESMM)
-// `extra` (may be null): one more addend of out's shape, added last (the gate path's share of an input gradient)
 template <typename T>
-__global__ __launch_bounds__(256) void sum_slots_kernel(T* __restrict__ out, const T* __restrict__ ws, int64_t n,
-                                                        int nws, const T* __restrict__ extra) {
-    constexpr int V = Vec16<T>::N;
-    const int64_t nv = n / V;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nv; i += stride) {
-        union { uint4 u; T e[V]; } o, w;
-        o.u = reinterpret_cast<const uint4*>(out)[i];
-        float acc[V];
-#pragma unroll
-        for (int j = 0; j < V; ++j) acc[j] = Cvt<T>::to_f(o.e[j]);
-        for (int s = 0; s < nws; ++s) {
-            w.u = reinterpret_cast<const uint4*>(ws + (size_t)s * n)[i];
-#pragma unroll
-            for (int j = 0; j < V; ++j) acc[j] += Cvt<T>::to_f(w.e[j]);
-        }
-        if (extra) {
-            w.u = reinterpret_cast<const uint4*>(extra)[i];
-#pragma unroll
-            for (int j = 0; j < V; ++j) acc[j] += Cvt<T>::to_f(w.e[j]);
-        }
-#pragma unroll
-        for (int j = 0; j < V; ++j) o.e[j] = Cvt<T>::from_f(acc[j]);
-        reinterpret_cast<uint4*>(out)[i] = o.u;
-    }
-}
+__global__ __launch_bounds__(256) void sum_slots_kernel(SumSlotsK p) { sum_slots_body<T>(p, blockIdx.x); }
 
 template <typename T>
-int launch_sum_slots_t(void* out, const void* ws, int64_t n, int nws, const void* extra, hipStream_t st) {
+int launch_sum_slots_t(void* out, const void* ws, int64_t n, int nws, const void* extra, int dt, hipStream_t st) {
     if (n == 0 || (nws == 0 && !extra)) return HEXA_OK;
     if (n % Vec16<T>::N) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "sum_slots: size must be a multiple of the vector width");
     int64_t blocks = (n / Vec16<T>::N + 255) / 256;
     if (blocks > 256 * 16) blocks = 256 * 16;
-    hipLaunchKernelGGL((sum_slots_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, (T*)out, (const T*)ws, n, nws,
-                       (const T*)extra);
-    HEXA_CHECK_LAUNCH("sum_slots");
+    SmallTask t;
+    t.kind = TASK_SUM_SLOTS; t.sum_slots = SumSlotsK{out, ws, n, nws, extra, (int)blocks}; t.blocks = (int)blocks;
+    if (!defer_task(defer_targets().sum_slots, t, dt)) {
+        hipLaunchKernelGGL((sum_slots_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, t.sum_slots);
+        HEXA_CHECK_LAUNCH("sum_slots");
+    }
     return HEXA_OK;
 }
 
 }  // namespace
 
 int launch_sum_slots(void* out, const void* ws, int64_t n, int nws, int dt, hipStream_t st, const void* extra) {
-    if (dt == HEXA_F32) return launch_sum_slots_t<float>(out, ws, n, nws, extra, st);
-    if (dt == HEXA_BF16) return launch_sum_slots_t<__bf16>(out, ws, n, nws, extra, st);
-    return launch_sum_slots_t<_Float16>(out, ws, n, nws, extra, st);
+    if (dt == HEXA_F32) return launch_sum_slots_t<float>(out, ws, n, nws, extra, dt, st);
+    if (dt == HEXA_BF16) return launch_sum_slots_t<__bf16>(out, ws, n, nws, extra, dt, st);
+    return launch_sum_slots_t<_Float16>(out, ws, n, nws, extra, dt, st);
 }
 
 int launch_ess(const EssArgs& a, hipStream_t st) {

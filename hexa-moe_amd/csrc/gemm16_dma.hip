@@ -28,6 +28,7 @@
 #include <algorithm>
 
 #include "dma_common.h"
+#include "small_bodies.h"
 
 namespace hexa {
 namespace {
@@ -289,48 +290,7 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
     }
 }
 
-// db[e][n] (+)= the column sums of expert e's row tiles, slot after slot, tile after tile (fixed order).
-// The tiles of a slot are listed expert after expert, so expert e's run starts at the number of tiles of the
-// experts before it: every thread of the workgroup adds up ceil(rows / tile_rows) over a share of those experts
-// (one round of loads instead of a bisection's chain of dependent ones).
-__global__ __launch_bounds__(256) void esmm_colsum_fold_kernel(void* __restrict__ db, const float* __restrict__ colsum,
-                                                               const int32_t* __restrict__ offsets, int E, int mt_ub,
-                                                               int tile_rows, int ntn, int bn, int N, int nslots,
-                                                               int db_dt, int accumulate) {
-    __shared__ int sFirst[8], sCount[8];        // per slot: first tile of expert e, its number of tiles
-    __shared__ int red[256];
-    const int e = blockIdx.y, tid = threadIdx.x;
-    for (int s = 0; s < nslots; ++s) {
-        const int32_t* off = offsets + (size_t)s * (E + 1);
-        int before = 0;
-        for (int x = tid; x < e; x += 256) before += (off[x + 1] - off[x] + tile_rows - 1) / tile_rows;
-        red[tid] = before;
-        __syncthreads();
-        for (int w = 128; w > 0; w >>= 1) {
-            if (tid < w) red[tid] += red[tid + w];
-            __syncthreads();
-        }
-        if (tid == 0) { sFirst[s] = red[0]; sCount[s] = (off[e + 1] - off[e] + tile_rows - 1) / tile_rows; }
-        __syncthreads();
-    }
-    const int n = blockIdx.x * 256 + tid;
-    if (n >= N) return;
-    const int nt = n / bn, nl = n - nt * bn;
-    float sum = 0.f;
-    for (int s = 0; s < nslots; ++s) {
-        const int first = sFirst[s], last = min(first + sCount[s], mt_ub);
-        // eight loads in flight per trip (a busy expert has a dozen tiles; one load per trip would pay the
-        // memory latency a dozen times); the additions stay in tile order
-        for (int mt = first; mt < last; mt += 8) {
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = colsum[(((size_t)s * mt_ub + min(mt + u, last - 1)) * ntn + nt) * bn + nl];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) sum += (mt + u < last) ? v[u] : 0.f;
-        }
-    }
-    store_out(db, (size_t)e * N + n, sum, db_dt, accumulate != 0);
-}
+__global__ __launch_bounds__(256) void esmm_colsum_fold_kernel(ColsumFoldK p) { colsum_fold_body(p, blockIdx.x); }
 
 template <typename TC, bool IO, bool OUT32, typename C>
 int launch_esmm_dma_t(EsmmK& p, int grid, hipStream_t st) {
@@ -365,80 +325,14 @@ struct EstmmK {
     float* scratch;
 };
 
-// ---- plan of a balanced ESTMM launch ------------------------------------------------------------------
-// One workgroup's walk over an expert's token list is serial, so the kernel is as slow as the
-// busiest expert.  With scratch memory, experts with more than `cap` tokens are cut into up to
-// PLAN_MAX_PARTS parts of equal step counts; a part is a unit of work like a whole small expert, its
-// fp32 partial result goes to a scratch slot, and estmm_fixup_kernel adds an expert's slots in order
-// (bit-reproducible).  Units are numbered heaviest expert first.  plan = 4 arrays of E ints in rank
-// order -- expert, parts, first unit, first scratch slot -- followed by the number of units.
-constexpr int PLAN_MAX_PARTS = 4;
-
+// The work plan (see small_bodies.h) as a launch of its own.
 __global__ __launch_bounds__(256) void estmm_plan_kernel(int* __restrict__ plan, const int32_t* __restrict__ offsets,
                                                          int E, int k, int cap, int max_slots) {
-    extern __shared__ int sp[];      // load[E], expert_of[E] (the expert at each rank)
-    int* load = sp;
-    int* expert_of = sp + E;
-    for (int e = threadIdx.x; e < E; e += 256) {
-        int t = 0;
-        for (int s = 0; s < k; ++s) t += offsets[(size_t)s * (E + 1) + e + 1] - offsets[(size_t)s * (E + 1) + e];
-        load[e] = t;
-    }
-    __syncthreads();
-    for (int e = threadIdx.x; e < E; e += 256) {
-        const int mine = load[e];
-        int r = 0;
-        for (int x = 0; x < E; ++x) {
-            const int o = load[x];
-            r += (o > mine || (o == mine && x < e)) ? 1 : 0;
-        }
-        expert_of[r] = e;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {          // E is small: a serial pass hands out units and scratch slots
-        int unit = 0, slot = 0;
-        for (int r = 0; r < E; ++r) {
-            const int e = expert_of[r];
-            int n = (load[e] + cap - 1) / cap;
-            n = max(1, min(n, PLAN_MAX_PARTS));
-            if (n > 1 && slot + n > max_slots) n = 1;
-            plan[r] = e;
-            plan[E + r] = n;
-            plan[2 * E + r] = unit;
-            plan[3 * E + r] = n > 1 ? slot : -1;
-            unit += n;
-            if (n > 1) slot += n;
-        }
-        plan[4 * E] = unit;
-    }
+    extern __shared__ int sp[];
+    estmm_plan_body(sp, plan, offsets, E, k, cap, max_slots);
 }
 
-// dw[e] (+)= slot[0] + slot[1] + ... for the experts that were cut into parts
-__global__ __launch_bounds__(256) void estmm_fixup_kernel(void* __restrict__ dw, const int* __restrict__ plan,
-                                                          const float* __restrict__ scratch, int E, long mn,
-                                                          int dw_dt, int accumulate) {
-    const int r = blockIdx.y;
-    const int n = plan[E + r];
-    if (n <= 1) return;
-    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i >= mn) return;
-    const int e = plan[r];
-    const float* src = scratch + (size_t)plan[3 * E + r] * mn + i;
-    // every part's load in flight at once (at most PLAN_MAX_PARTS), added in part order
-    float4 w[PLAN_MAX_PARTS];
-#pragma unroll
-    for (int c = 0; c < PLAN_MAX_PARTS; ++c) w[c] = *reinterpret_cast<const float4*>(src + (size_t)min(c, n - 1) * mn);
-    float4 v = w[0];
-#pragma unroll
-    for (int c = 1; c < PLAN_MAX_PARTS; ++c) {
-        if (c < n) { v.x += w[c].x; v.y += w[c].y; v.z += w[c].z; v.w += w[c].w; }
-    }
-    const size_t o = (size_t)e * mn + i;
-    store_out(dw, o, v.x, dw_dt, accumulate != 0);
-    store_out(dw, o + 1, v.y, dw_dt, accumulate != 0);
-    store_out(dw, o + 2, v.z, dw_dt, accumulate != 0);
-    store_out(dw, o + 3, v.w, dw_dt, accumulate != 0);
-}
+__global__ __launch_bounds__(256) void estmm_fixup_kernel(FixupK p) { estmm_fixup_body(p, blockIdx.x); }
 
 struct Cursor {   // walks the expert's token list in 32-token steps, slot after slot
     int s, r;
@@ -713,9 +607,14 @@ int launch_estmm_dma_c(const EstmmArgs& a, hipStream_t st) {
     if (a.pq_dt == HEXA_BF16) rc = o32 ? launch_estmm_dma_t<__bf16, true, C>(p, grid, st) : launch_estmm_dma_t<__bf16, false, C>(p, grid, st);
     else rc = o32 ? launch_estmm_dma_t<_Float16, true, C>(p, grid, st) : launch_estmm_dma_t<_Float16, false, C>(p, grid, st);
     if (rc || !p.plan) return rc;
-    hipLaunchKernelGGL(estmm_fixup_kernel, dim3((unsigned)((mn / 4 + 255) / 256), E), dim3(256), 0, st, a.dw, p.plan, p.scratch,
-                       E, mn, a.dw_dt, a.accumulate);
-    HEXA_CHECK_LAUNCH("estmm_fixup");
+    SmallTask t;
+    t.kind = TASK_FIXUP;
+    t.fixup = FixupK{a.dw, p.plan, p.scratch, E, mn, a.dw_dt, a.accumulate, (int)((mn / 4 + 255) / 256)};
+    t.blocks = t.fixup.gx * E;
+    if (!defer_task(defer_targets().fixup, t)) {
+        hipLaunchKernelGGL(estmm_fixup_kernel, dim3(t.blocks), dim3(256), 0, st, t.fixup);
+        HEXA_CHECK_LAUNCH("estmm_fixup");
+    }
     return HEXA_OK;
 }
 
@@ -778,18 +677,22 @@ int pick_esmm_tile(long rows, int cols, int in_dim) {
 }  // namespace
 
 int launch_colsum_fold(const EsmmArgs& a, int mt_ub, int tile_rows, int ntn, int bn, hipStream_t st) {
-    hipLaunchKernelGGL(esmm_colsum_fold_kernel, dim3(div_up(a.out_dim, 256), a.r.E), dim3(256), 0, st, a.db, a.colsum, a.r.offsets,
-                       a.r.E, mt_ub, tile_rows, ntn, bn, a.out_dim, a.r.k, a.db_dt, a.db_accumulate);
-    HEXA_CHECK_LAUNCH("esmm_colsum_fold");
+    SmallTask t;
+    t.kind = TASK_COLSUM_FOLD;
+    t.colsum_fold = ColsumFoldK{a.db, a.colsum, a.r.offsets, a.r.E, mt_ub, tile_rows, ntn, bn, a.out_dim, a.r.k, a.db_dt,
+                                a.db_accumulate, div_up(a.out_dim, 256)};
+    t.blocks = t.colsum_fold.gx * a.r.E;
+    if (!defer_task(defer_targets().colsum_fold, t)) {
+        hipLaunchKernelGGL(esmm_colsum_fold_kernel, dim3(t.blocks), dim3(256), 0, st, t.colsum_fold);
+        HEXA_CHECK_LAUNCH("esmm_colsum_fold");
+    }
     return HEXA_OK;
 }
 
 int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, hipStream_t st) {
     if (r.E > 4096) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "estmm plan: more than 4096 experts");
-    const long avg = (long)r.T * r.k / r.E;
-    const int cap = (int)std::max<long>(256, (3 * avg + 1) / 2);   // parts for experts above 1.5x the mean load
-    hipLaunchKernelGGL(estmm_plan_kernel, dim3(1), dim3(256), 3 * r.E * sizeof(int), st, plan, r.offsets, r.E, r.k, cap,
-                       max_slots);
+    hipLaunchKernelGGL(estmm_plan_kernel, dim3(1), dim3(256), 2 * r.E * sizeof(int), st, plan, r.offsets, r.E, r.k,
+                       estmm_plan_cap(r.T, r.k, r.E), max_slots);
     HEXA_CHECK_LAUNCH("estmm_plan");
     return HEXA_OK;
 }

@@ -94,6 +94,7 @@ enum Opt {
     OPT_ESTMM_GROUP,    // HEXA_ESTMM_GROUP: row tiles per XCD run
     OPT_ESMM_STREAM,    // HEXA_ESMM_STREAM: 1 = results stored with the streaming hint
     OPT_ROUTE_KERNELS,  // HEXA_ROUTE_KERNELS: 3 = always the three-launch routing pass, 1 = one launch up to 65536 tokens
+    OPT_BATCH,          // HEXA_MOE_BATCH: 2 = every small kernel of the depth backward in a launch of its own
     OPT_FFN_FUSED,      // HEXA_MOE_FFN_FUSED: 1 = hexa_moe_depth_forward runs fc1, GELU and fc2 in one kernel where it is covered
     OPT_COUNT
 };
@@ -118,6 +119,16 @@ int launch_estmm32(const EstmmArgs& a, hipStream_t s);
 int launch_ess(const EssArgs& a, hipStream_t s);
 int launch_ess_noalloc(EssArgs a, hipStream_t s);
 int launch_sum_slots(void* out, const void* ws, int64_t n, int nws, int dt, hipStream_t s, const void* extra = nullptr);
+// routing front end of the depth call: the router also counts, the counting sort's scan launch also finishes the loss,
+// its scatter launch also makes the ESTMM plan (see router.hip, route.hip)
+bool router_hist_supported(int E);
+int router_tokens_per_workgroup();
+int router_forward_check(int T, int E, int k, bool ptrs_ok);
+int launch_router_fwd(float* scores, int32_t* idx, const float* logits, const float* noise, float noise_scale, int T, int E,
+                      int k, float* ws, int32_t* hist, hipStream_t st);
+int launch_route_from_hist(const int32_t* idx, int T, int k, int E, int32_t* route, int32_t* hist, int unit_tokens,
+                           float* l_aux, float* me, float* ce, const float* router_ws, int32_t* plan, int plan_slots,
+                           hipStream_t st);
 int launch_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, hipStream_t s);
 
 // ---- small device helpers -------------------------------------------------------------------

@@ -10,7 +10,10 @@
 // Replaces launch_count / launch_assign of the reference (kernels/shared_cuda_core.cu:126-182,
 // 284-333), which run single-workgroup launches with shared-memory atomics, two blocking copies and
 // a host-side prefix per call.
+#include <algorithm>
+
 #include "hexa_internal.h"
+#include "small_bodies.h"
 
 namespace hexa {
 namespace {
@@ -124,20 +127,15 @@ __device__ void finish_slot(const int32_t* tot, int32_t* off, int32_t* tbase, in
 // One workgroup per slot.  Turns unit_hist[s][u][e] into the exclusive prefix over u (in place) and
 // finishes the slot.  given_offsets != nullptr: legacy TOKEN_ASSIGN, segment starts come from the
 // caller and nothing but the unit prefixes is written.
-__global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ unit_hist, int E, int units,
-                                                         int pad, int32_t* __restrict__ counts,
-                                                         int32_t* __restrict__ offsets,
-                                                         int4* __restrict__ tile_info,
-                                                         int32_t* __restrict__ tile_count, int mt_ub,
-                                                         int4* __restrict__ tile_info_l,
-                                                         int32_t* __restrict__ tile_count_l, int mt_ub_l,
-                                                         int prefix_only) {
-    extern __shared__ int32_t sh[];
+__device__ __forceinline__ void route_scan_body(int32_t* sh, int s, int32_t* __restrict__ unit_hist, int E, int units,
+                                                int pad, int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
+                                                int4* __restrict__ tile_info, int32_t* __restrict__ tile_count, int mt_ub,
+                                                int4* __restrict__ tile_info_l, int32_t* __restrict__ tile_count_l,
+                                                int mt_ub_l, int prefix_only) {
     int32_t* tot = sh;
     int32_t* off = tot + E;
     int32_t* tbase = off + (E + 1);
     int* tmp = tbase + (E + 1);
-    const int s = blockIdx.x;
     int32_t* H = unit_hist + (size_t)s * units * E;
     // Exclusive prefix over the units, per expert.  Up to 256 experts: 256/E threads share an expert,
     // each takes a contiguous range of units (sum, then rewrite), and loads go 8 at a time so that the
@@ -151,14 +149,24 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ u
         const bool active = e < E && j < G;
         const int per = (units + G - 1) / G;
         const int u_begin = min(units, j * per), u_end = min(units, u_begin + per);
+        // up to SCAN_KEEP units per thread stay in registers between the sum and the rewrite: all of a thread's
+        // loads are in flight at once and nothing is read twice
+        constexpr int SCAN_KEEP = 40;
+        const bool keep = per <= SCAN_KEEP;
+        int c[SCAN_KEEP];
         int sum = 0;
-        if (active) {
+        if (active && keep) {
+#pragma unroll
+            for (int i = 0; i < SCAN_KEEP; ++i) c[i] = u_begin + i < u_end ? H[(size_t)(u_begin + i) * E + e] : 0;
+#pragma unroll
+            for (int i = 0; i < SCAN_KEEP; ++i) sum += c[i];
+        } else if (active) {
             for (int u0 = u_begin; u0 < u_end; u0 += 8) {
-                int c[8];
+                int v[8];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) c[i] = u0 + i < u_end ? H[(size_t)(u0 + i) * E + e] : 0;
+                for (int i = 0; i < 8; ++i) v[i] = u0 + i < u_end ? H[(size_t)(u0 + i) * E + e] : 0;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) sum += c[i];
+                for (int i = 0; i < 8; ++i) sum += v[i];
             }
         }
         if (G > 1) {
@@ -175,14 +183,22 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ u
             } else if (G == 1) {
                 tot[e] = sum;
             }
-            for (int u0 = u_begin; u0 < u_end; u0 += 8) {
-                int c[8];
+            if (keep) {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) c[i] = u0 + i < u_end ? H[(size_t)(u0 + i) * E + e] : 0;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    if (u0 + i < u_end) H[(size_t)(u0 + i) * E + e] = run;
+                for (int i = 0; i < SCAN_KEEP; ++i) {
+                    if (u_begin + i < u_end) H[(size_t)(u_begin + i) * E + e] = run;
                     run += c[i];
+                }
+            } else {
+                for (int u0 = u_begin; u0 < u_end; u0 += 8) {
+                    int v[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) v[i] = u0 + i < u_end ? H[(size_t)(u0 + i) * E + e] : 0;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        if (u0 + i < u_end) H[(size_t)(u0 + i) * E + e] = run;
+                        run += v[i];
+                    }
                 }
             }
         }
@@ -197,24 +213,55 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ u
                 tile_count_l ? tile_count_l + s : nullptr, mt_ub_l);
 }
 
+__global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ unit_hist, int E, int units,
+                                                         int pad, int32_t* __restrict__ counts,
+                                                         int32_t* __restrict__ offsets,
+                                                         int4* __restrict__ tile_info,
+                                                         int32_t* __restrict__ tile_count, int mt_ub,
+                                                         int4* __restrict__ tile_info_l,
+                                                         int32_t* __restrict__ tile_count_l, int mt_ub_l,
+                                                         int prefix_only) {
+    extern __shared__ int32_t sh[];
+    route_scan_body(sh, blockIdx.x, unit_hist, E, units, pad, counts, offsets, tile_info, tile_count, mt_ub, tile_info_l,
+                    tile_count_l, mt_ub_l, prefix_only);
+}
+
+// The scan of every slot (workgroups 0..k-1) and, in one more workgroup of the same launch, the GShard loss from
+// the router's partial sums: the two do not depend on each other, and a launch of its own for a single small
+// workgroup costs as much as the whole scan.
+__global__ __launch_bounds__(256) void route_scan_loss_kernel(int32_t* __restrict__ unit_hist, int E, int units, int k,
+                                                              int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
+                                                              int4* __restrict__ tile_info,
+                                                              int32_t* __restrict__ tile_count, int mt_ub,
+                                                              int4* __restrict__ tile_info_l,
+                                                              int32_t* __restrict__ tile_count_l, int mt_ub_l,
+                                                              float* __restrict__ l_aux, float* __restrict__ me,
+                                                              float* __restrict__ ce, const float* __restrict__ part_me,
+                                                              const float* __restrict__ part_cnt, int nblocks,
+                                                              int num_tokens) {
+    extern __shared__ int32_t sh[];
+    if ((int)blockIdx.x < k)
+        route_scan_body(sh, blockIdx.x, unit_hist, E, units, 1, counts, offsets, tile_info, tile_count, mt_ub, tile_info_l,
+                        tile_count_l, mt_ub_l, 0);
+    else
+        router_loss_body(reinterpret_cast<float*>(sh), l_aux, me, ce, part_me, part_cnt, nblocks, num_tokens, E);
+}
+
 template <typename IdxT>
-__global__ __launch_bounds__(kWave) void route_scatter_kernel(const IdxT* __restrict__ routing,
-                                                              int64_t token_stride, int64_t slot_stride,
-                                                              int T, int E, int units, int nbits,
-                                                              const int32_t* __restrict__ unit_hist,
-                                                              const int32_t* __restrict__ offsets,
-                                                              int64_t offsets_slot_stride,
-                                                              int32_t* __restrict__ token_ids,
-                                                              int32_t* __restrict__ expert_ids,
-                                                              int64_t list_stride) {
-    extern __shared__ int32_t cursor[];
-    const int lane = threadIdx.x, unit = blockIdx.x, s = blockIdx.y;
+__device__ __forceinline__ void route_scatter_body(int32_t* cursor, int unit, int s, int unit_tokens,
+                                                   const IdxT* __restrict__ routing, int64_t token_stride,
+                                                   int64_t slot_stride, int T, int E, int units, int nbits,
+                                                   const int32_t* __restrict__ unit_hist,
+                                                   const int32_t* __restrict__ offsets, int64_t offsets_slot_stride,
+                                                   int32_t* __restrict__ token_ids, int32_t* __restrict__ expert_ids,
+                                                   int64_t list_stride) {
+    const int lane = threadIdx.x;
     const int32_t* H = unit_hist + ((size_t)s * units + unit) * E;
     const int32_t* off = offsets + (size_t)s * offsets_slot_stride;
     for (int i = lane; i < E; i += kWave) cursor[i] = off[i] + H[i];
     __syncthreads();
-    const int t0 = unit * kUnit;
-    const int t1 = min(T, t0 + kUnit);
+    const int t0 = unit * unit_tokens;
+    const int t1 = min(T, t0 + unit_tokens);
     const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
     int32_t* tok = token_ids + (size_t)s * list_stride;
     int32_t* exp = expert_ids ? expert_ids + (size_t)s * list_stride : nullptr;
@@ -239,6 +286,40 @@ __global__ __launch_bounds__(kWave) void route_scatter_kernel(const IdxT* __rest
             if ((peers & lt_mask) == 0) cursor[e] += __popcll(peers);  // first lane of its group
         }
         __syncthreads();
+    }
+}
+
+template <typename IdxT>
+__global__ __launch_bounds__(kWave) void route_scatter_kernel(const IdxT* __restrict__ routing,
+                                                              int64_t token_stride, int64_t slot_stride,
+                                                              int T, int E, int units, int nbits,
+                                                              const int32_t* __restrict__ unit_hist,
+                                                              const int32_t* __restrict__ offsets,
+                                                              int64_t offsets_slot_stride,
+                                                              int32_t* __restrict__ token_ids,
+                                                              int32_t* __restrict__ expert_ids,
+                                                              int64_t list_stride) {
+    extern __shared__ int32_t cursor[];
+    route_scatter_body<IdxT>(cursor, blockIdx.x, blockIdx.y, kUnit, routing, token_stride, slot_stride, T, E, units, nbits,
+                             unit_hist, offsets, offsets_slot_stride, token_ids, expert_ids, list_stride);
+}
+
+// The scatter over units of `unit_tokens` tokens of a [T][k] int32 routing table and, in one more workgroup of the
+// same launch (x = units, y = 0), the work plan of the balanced ESTMM, which needs nothing but the offsets.
+__global__ __launch_bounds__(kWave) void route_scatter_plan_kernel(const int32_t* __restrict__ routing, int k, int T, int E,
+                                                                   int units, int unit_tokens, int nbits,
+                                                                   const int32_t* __restrict__ unit_hist,
+                                                                   const int32_t* __restrict__ offsets,
+                                                                   int32_t* __restrict__ token_ids,
+                                                                   int32_t* __restrict__ expert_ids,
+                                                                   int32_t* __restrict__ plan, int plan_cap,
+                                                                   int plan_slots) {
+    extern __shared__ int32_t cursor[];
+    if ((int)blockIdx.x < units) {
+        route_scatter_body<int32_t>(cursor, blockIdx.x, blockIdx.y, unit_tokens, routing, k, 1, T, E, units, nbits, unit_hist,
+                                    offsets, E + 1, token_ids, expert_ids, T);
+    } else if (blockIdx.y == 0 && plan) {
+        estmm_plan_body(cursor, plan, offsets, E, k, plan_cap, plan_slots);
     }
 }
 
@@ -452,6 +533,30 @@ RouteView route_view(const int32_t* route, int T, int k, int E) {
     v.tile_count_l = route + L.tile_count_l;
     v.T = T; v.k = k; v.E = E; v.mt_ub = L.mt_ub; v.mt_ub_l = L.mt_ub_l;
     return v;
+}
+}  // namespace hexa
+
+namespace hexa {
+// The routing pass for a [T][k] int32 table whose histogram over units of `unit_tokens` tokens (hist [k][units][E])
+// has been counted already: scan (+ the GShard loss, when l_aux is given, from the router's partial sums in
+// router_ws) and scatter (+ the ESTMM work plan, when plan is given).
+int launch_route_from_hist(const int32_t* idx, int T, int k, int E, int32_t* route, int32_t* hist, int unit_tokens,
+                           float* l_aux, float* me, float* ce, const float* router_ws, int32_t* plan, int plan_slots,
+                           hipStream_t st) {
+    hexa_route_layout L;
+    hexa_route_layout_get(T, k, E, &L);
+    const int units = div_up(T, unit_tokens);
+    const size_t loss_lds = l_aux ? sizeof(float) * (2 * (size_t)router_loss_chunks(E) * E + 256) : 0;
+    hipLaunchKernelGGL(route_scan_loss_kernel, dim3(k + (l_aux ? 1 : 0)), dim3(256), std::max(scan_lds_bytes(E), loss_lds), st,
+                       hist, E, units, k, route + L.counts, route + L.offsets, reinterpret_cast<int4*>(route + L.tile_info),
+                       route + L.tile_count, L.mt_ub, reinterpret_cast<int4*>(route + L.tile_info_l), route + L.tile_count_l,
+                       L.mt_ub_l, l_aux, me, ce, router_ws, router_ws ? router_ws + (size_t)units * E : nullptr, units, T);
+    HEXA_CHECK_LAUNCH("route_scan_loss");
+    hipLaunchKernelGGL(route_scatter_plan_kernel, dim3(units + (plan ? 1 : 0), k), dim3(kWave), sizeof(int32_t) * 2 * E, st, idx,
+                       k, T, E, units, unit_tokens, ceil_log2(E), hist, route + L.offsets, route + L.token_ids,
+                       route + L.expert_ids, plan, estmm_plan_cap(T, k, E), plan_slots);
+    HEXA_CHECK_LAUNCH("route_scatter_plan");
+    return HEXA_OK;
 }
 }  // namespace hexa
 

@@ -7,6 +7,7 @@
 //            hexa_moe_cuda/hexa_moe/impls/cascaded_moe.py:515-531 (noise, softmax, loss selection),
 //            hexa_moe_cuda/hexa_moe/impls/layers.py:476-484 (top-k), impls/losses.py:12-19 (GShard loss).
 #include "hexa_internal.h"
+#include "small_bodies.h"
 
 namespace hexa {
 namespace {
@@ -99,17 +100,23 @@ __host__ __device__ constexpr int router_pitch(int E) {
     return 4 * p;
 }
 
+// hist (optional): [k][workgroups][E] ints, per slot the number of this workgroup's 64 tokens that chose each expert
+// -- the histogram the routing pass starts from (units of 64 tokens), so that pass needs no counting launch.
 __global__ __launch_bounds__(ROUTER_TB * ROUTER_G) void router_fwd4_kernel(
     float* __restrict__ scores, int32_t* __restrict__ idx, float* __restrict__ part_me, float* __restrict__ part_cnt,
-    const float* __restrict__ logits, const float* __restrict__ noise, float noise_scale, int num_tokens, int E, int k) {
-    extern __shared__ float sh[];          // cnt[E], then the tile [64][P]
+    const float* __restrict__ logits, const float* __restrict__ noise, float noise_scale, int num_tokens, int E, int k,
+    int32_t* __restrict__ hist) {
+    extern __shared__ float sh[];          // cnt[E], the tile [64][P], then hist[k][E]
     float* s_cnt = sh;
     const int P = router_pitch(E);
     float* tile = sh + ((E + 3) & ~3);
+    int* s_hist = reinterpret_cast<int*>(tile + ROUTER_TB * P);
     const int tid = threadIdx.x;
     const int t0 = blockIdx.x * ROUTER_TB;
     const int rows = min(ROUTER_TB, num_tokens - t0);
     for (int i = tid; i < E; i += blockDim.x) s_cnt[i] = 0.f;
+    if (hist)
+        for (int i = tid; i < k * E; i += blockDim.x) s_hist[i] = 0;
     // ---- tile in: element i of the contiguous block [rows][E] ----
     const size_t g0 = (size_t)t0 * E;
     const int total = rows * E;
@@ -192,7 +199,10 @@ __global__ __launch_bounds__(ROUTER_TB * ROUTER_G) void router_fwd4_kernel(
     if (ok) {
 #pragma unroll
         for (int j = 0; j < MAX_TOPK; ++j)
-            if (j < k && (j & 3) == q) idx[(size_t)t * k + j] = pick[j];
+            if (j < k && (j & 3) == q) {
+                idx[(size_t)t * k + j] = pick[j];
+                if (hist) atomicAdd(&s_hist[j * E + pick[j]], 1);
+            }
         if (q == 0) atomicAdd(&s_cnt[pick[0]], 1.0f);   // exact: at most 64 ones per counter
     }
     __syncthreads();
@@ -204,6 +214,11 @@ __global__ __launch_bounds__(ROUTER_TB * ROUTER_G) void router_fwd4_kernel(
         part_me[(size_t)blockIdx.x * E + e] = m;
         part_cnt[(size_t)blockIdx.x * E + e] = s_cnt[e];
     }
+    if (hist)
+        for (int i = tid; i < k * E; i += blockDim.x) {
+            const int j = i / E, e = i - j * E;
+            hist[((size_t)j * gridDim.x + blockIdx.x) * E + e] = s_hist[i];
+        }
     if ((E & 3) == 0) {
         for (int i = tid * 4; i < total; i += blockDim.x * 4) {
             const int rr = i / E, e = i - rr * E;
@@ -217,88 +232,18 @@ __global__ __launch_bounds__(ROUTER_TB * ROUTER_G) void router_fwd4_kernel(
     }
 }
 
-// me[e] = sum_t scores[t][e]; ce[e] = count[e] * E / T; l_aux = sum_e me[e]*ce[e] / T  (losses.py:12-19)
+// The GShard loss from the workgroup partials (see small_bodies.h) as a launch of its own.
 __global__ __launch_bounds__(256) void router_loss_kernel(float* __restrict__ l_aux, float* __restrict__ me,
                                                           float* __restrict__ ce, const float* __restrict__ part_me,
                                                           const float* __restrict__ part_cnt, int nblocks,
                                                           int num_tokens, int E) {
-    // per expert: nch threads sum nch contiguous ranges of the workgroup partials, then the range sums
-    // are added in range order -- a fixed tree, independent of scheduling
-    extern __shared__ float sh[];          // [nch][E] me, [nch][E] cnt
-    const int nch = max(1, min(32, 8192 / E));
-    float* s_m = sh;
-    float* s_c = sh + nch * E;
-    __shared__ float red[256];
-    const int per = (nblocks + nch - 1) / nch;
-    for (int i = threadIdx.x; i < nch * E; i += 256) {
-        const int c = i / E, e = i - c * E;
-        const int b0 = c * per, b1 = min(nblocks, b0 + per);
-        float m = 0.f, n = 0.f;
-        for (int b = b0; b < b1; b += 8) {     // eight partials of each kind in flight per trip, added in order
-            float pm[8], pc[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const size_t at = (size_t)min(b + u, b1 - 1) * E + e;
-                pm[u] = part_me[at];
-                pc[u] = part_cnt[at];
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                m += (b + u < b1) ? pm[u] : 0.f;
-                n += (b + u < b1) ? pc[u] : 0.f;
-            }
-        }
-        s_m[i] = m;
-        s_c[i] = n;
-    }
-    __syncthreads();
-    float local = 0.f;
-    for (int e = threadIdx.x; e < E; e += 256) {
-        float m = 0.f, c = 0.f;
-        for (int j = 0; j < nch; ++j) { m += s_m[j * E + e]; c += s_c[j * E + e]; }
-        const float cev = c * ((float)E / (float)num_tokens);
-        me[e] = m;
-        ce[e] = cev;
-        local += m * cev;
-    }
-    red[threadIdx.x] = local;
-    __syncthreads();
-    for (int s = 128; s > 0; s >>= 1) {
-        if (threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) *l_aux = red[0] / (float)num_tokens;
+    extern __shared__ float sh[];
+    router_loss_body(sh, l_aux, me, ce, part_me, part_cnt, nblocks, num_tokens, E);
 }
 
-// d l_aux / d logits through the softmax: with c[e] = g * ce[e] / T,
-//   dlogits[t][e] = scores[t][e] * (c[e] - sum_e' scores[t][e'] * c[e'])
-__global__ __launch_bounds__(ROUTER_TB) void router_bwd_kernel(float* __restrict__ dlogits,
-                                                               const float* __restrict__ scores,
-                                                               const float* __restrict__ ce,
-                                                               const float* __restrict__ grad_l, int num_tokens, int E) {
-    extern __shared__ float s_c[];         // c[e] = g * ce[e] / T
-    const float g = *grad_l / (float)num_tokens;
-    for (int e = threadIdx.x; e < E; e += blockDim.x) s_c[e] = g * ce[e];
-    __syncthreads();
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= num_tokens) return;
-    const float* sr = scores + (size_t)t * E;
-    float* dr = dlogits + (size_t)t * E;
-    float dot = 0.f;
-    if ((E & 3) == 0) {
-        for (int e = 0; e < E; e += 4) {
-            const float4 v = *reinterpret_cast<const float4*>(sr + e);
-            dot += v.x * s_c[e] + v.y * s_c[e + 1] + v.z * s_c[e + 2] + v.w * s_c[e + 3];
-        }
-        for (int e = 0; e < E; e += 4) {
-            const float4 v = *reinterpret_cast<const float4*>(sr + e);
-            *reinterpret_cast<float4*>(dr + e) = make_float4(v.x * (s_c[e] - dot), v.y * (s_c[e + 1] - dot),
-                                                             v.z * (s_c[e + 2] - dot), v.w * (s_c[e + 3] - dot));
-        }
-    } else {
-        for (int e = 0; e < E; ++e) dot += sr[e] * s_c[e];
-        for (int e = 0; e < E; ++e) dr[e] = sr[e] * (s_c[e] - dot);
-    }
+__global__ __launch_bounds__(256) void router_bwd_kernel(RouterBwdK p) {
+    extern __shared__ float s_c[];
+    router_bwd_body(s_c, p, blockIdx.x);
 }
 
 
@@ -489,27 +434,50 @@ extern "C" int hexa_router_ws_floats(int T, int E, int64_t* out) {
     return HEXA_OK;
 }
 
-extern "C" int hexa_router_forward(float* scores, int32_t* idx, float* me, float* ce, float* l_aux,
-                                   const float* logits, const float* noise, float noise_scale, int T, int E, int k,
-                                   float* ws, void* stream) {
-    if (T < 1 || E < 1 || k < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_router_forward: bad sizes T=%d E=%d k=%d", T, E, k);
-    if (k > MAX_TOPK || k > E) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_router_forward: top_k must be <= min(E, %d)", MAX_TOPK);
-    if (!scores || !idx || !me || !ce || !l_aux || !logits || !ws) HEXA_FAIL(HEXA_ERR_ARG, "hexa_router_forward: null pointer");
-    if (E > 4096) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_router_forward: more than 4096 experts");
-    hipStream_t st = (hipStream_t)stream;
+namespace hexa {
+bool router_hist_supported(int E) { return E <= ROUTER_LDS_E; }
+int router_tokens_per_workgroup() { return ROUTER_TB; }
+
+// softmax + top-k + the loss partials (ws: hexa_router_ws_floats() floats); with `hist` (only where
+// router_hist_supported) also the routing pass's histogram over units of 64 tokens
+int launch_router_fwd(float* scores, int32_t* idx, const float* logits, const float* noise, float noise_scale, int T, int E,
+                      int k, float* ws, int32_t* hist, hipStream_t st) {
     const int nb = div_up(T, ROUTER_TB);
     float* part_me = ws;
     float* part_cnt = ws + (size_t)nb * E;
     if (E <= ROUTER_LDS_E)
-        hipLaunchKernelGGL(router_fwd4_kernel, dim3(nb), dim3(ROUTER_TB * ROUTER_G), sizeof(float) * (((E + 3) & ~3) + ROUTER_TB * router_pitch(E)),
-                           st, scores, idx, part_me, part_cnt, logits, noise, noise_scale, T, E, k);
+        hipLaunchKernelGGL(router_fwd4_kernel, dim3(nb), dim3(ROUTER_TB * ROUTER_G),
+                           sizeof(float) * (((E + 3) & ~3) + ROUTER_TB * router_pitch(E) + (hist ? k * E : 0)), st, scores, idx,
+                           part_me, part_cnt, logits, noise, noise_scale, T, E, k, hist);
     else
         hipLaunchKernelGGL(router_fwd_kernel, dim3(nb), dim3(ROUTER_TB), sizeof(float) * 2 * E, st, scores, idx,
                            part_me, part_cnt, logits, noise, noise_scale, T, E, k);
     HEXA_CHECK_LAUNCH("router_fwd");
-    const int nch = E <= 256 ? 32 : (8192 / E > 0 ? 8192 / E : 1);
-    hipLaunchKernelGGL(router_loss_kernel, dim3(1), dim3(256), sizeof(float) * 2 * nch * E, st, l_aux, me, ce, part_me,
-                       part_cnt, nb, T, E);
+    return HEXA_OK;
+}
+}  // namespace hexa
+
+static int check_router_forward(int T, int E, int k, bool ptrs_ok) {
+    if (T < 1 || E < 1 || k < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_router_forward: bad sizes T=%d E=%d k=%d", T, E, k);
+    if (k > MAX_TOPK || k > E) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_router_forward: top_k must be <= min(E, %d)", MAX_TOPK);
+    if (!ptrs_ok) HEXA_FAIL(HEXA_ERR_ARG, "hexa_router_forward: null pointer");
+    if (E > 4096) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_router_forward: more than 4096 experts");
+    return HEXA_OK;
+}
+
+namespace hexa {
+int router_forward_check(int T, int E, int k, bool ptrs_ok) { return check_router_forward(T, E, k, ptrs_ok); }
+}
+
+extern "C" int hexa_router_forward(float* scores, int32_t* idx, float* me, float* ce, float* l_aux,
+                                   const float* logits, const float* noise, float noise_scale, int T, int E, int k,
+                                   float* ws, void* stream) {
+    if (int rc = check_router_forward(T, E, k, scores && idx && me && ce && l_aux && logits && ws)) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    if (int rc = launch_router_fwd(scores, idx, logits, noise, noise_scale, T, E, k, ws, nullptr, st)) return rc;
+    const int nb = div_up(T, ROUTER_TB);
+    hipLaunchKernelGGL(router_loss_kernel, dim3(1), dim3(256), sizeof(float) * (2 * router_loss_chunks(E) * E + 256), st,
+                       l_aux, me, ce, ws, ws + (size_t)nb * E, nb, T, E);
     HEXA_CHECK_LAUNCH("router_loss");
     return HEXA_OK;
 }
@@ -519,9 +487,12 @@ extern "C" int hexa_router_backward(float* dlogits, const float* scores, const f
     if (T < 1 || E < 1) HEXA_FAIL(HEXA_ERR_ARG, "hexa_router_backward: bad sizes");
     if (!dlogits || !scores || !ce || !grad_l_aux) HEXA_FAIL(HEXA_ERR_ARG, "hexa_router_backward: null pointer");
     if (E > 8192) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "hexa_router_backward: more than 8192 experts");
-    hipLaunchKernelGGL(router_bwd_kernel, dim3(div_up(T, ROUTER_TB)), dim3(ROUTER_TB), sizeof(float) * E,
-                       (hipStream_t)stream, dlogits, scores, ce, grad_l_aux, T, E);
-    HEXA_CHECK_LAUNCH("router_bwd");
+    SmallTask t;
+    t.kind = TASK_ROUTER_BWD; t.router_bwd = RouterBwdK{dlogits, scores, ce, grad_l_aux, T, E}; t.blocks = div_up(T, 256);
+    if (!defer_task(E <= BATCH_ROUTER_BWD_MAX_E ? defer_targets().router_bwd : nullptr, t)) {
+        hipLaunchKernelGGL(router_bwd_kernel, dim3(t.blocks), dim3(256), sizeof(float) * E, (hipStream_t)stream, t.router_bwd);
+        HEXA_CHECK_LAUNCH("router_bwd");
+    }
     return HEXA_OK;
 }
 

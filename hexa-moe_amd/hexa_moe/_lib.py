@@ -62,8 +62,8 @@ SIGNATURES = {
                                                  ctypes.c_float, _i, _i, _i, _vp, _vp]),
     "hexa_router_backward_load_importance": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float, _i, _i, _i, _vp]),
     "hexa_moe_depth_ws_bytes": (_i, [ctypes.POINTER(DepthDesc), ctypes.POINTER(_i64), ctypes.POINTER(_i64)]),
-    "hexa_moe_depth_forward": (_i, [ctypes.POINTER(DepthDesc)] + [_vp] * 16 + [_vp, _i64, _vp, _i, _vp]),
-    "hexa_moe_depth_backward": (_i, [ctypes.POINTER(DepthDesc)] + [_vp] * 20 + [_vp, _i64, _vp, _i, _vp]),
+    "hexa_moe_depth_forward": (_i, [ctypes.POINTER(DepthDesc)] + [_vp] * 17 + [_vp, _i64, _vp, _i, _vp]),
+    "hexa_moe_depth_backward": (_i, [ctypes.POINTER(DepthDesc)] + [_vp] * 21 + [_vp, _i64, _vp, _i, _vp]),
     "hexa_last_error": (ctypes.c_char_p, []),
     "hexa_abi_version": (_i, []),
     "hexa_set_option": (_i, [ctypes.c_char_p, _i]),
@@ -86,7 +86,7 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.hexa_abi_version() != 7:
+    if lib.hexa_abi_version() != 8:
         raise RuntimeError("hexa_moe: libhexa_moe_hip.so has an unexpected ABI version")
     _lib = lib
     return lib

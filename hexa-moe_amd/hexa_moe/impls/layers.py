@@ -216,7 +216,8 @@ class FusedMoEDepth(torch.autograd.Function):
         state = torch.empty(2 * T * E + T + nstats, dtype=torch.float32, device=dev)
         logits, scores = state[:T * E], state[T * E:2 * T * E]
         thr, stats = state[2 * T * E:2 * T * E + T], state[2 * T * E + T:]
-        idx = torch.empty(T, top_k, dtype=torch.int32, device=dev)
+        ints = torch.empty(T * top_k + 4 * E + 1, dtype=torch.int32, device=dev)
+        idx, estmm_plan = ints[:T * top_k].view(T, top_k), ints[T * top_k:]   # the backward's ESTMM work plan: 4E+1 ints
         noise = torch.randn(T, E, dtype=torch.float32, device=dev) if noise_scale > 0 else None
         blob = config.route_pool.slot(config.stage, T, top_k, E, dev)
         y12 = torch.empty(2, top_k, T, hidden, dtype=x.dtype, device=dev)
@@ -224,7 +225,7 @@ class FusedMoEDepth(torch.autograd.Function):
         ws = torch.empty(plan.fwd_bytes, dtype=torch.uint8, device=dev)
         ev = FusedMoEDepth.events
         ops.moe_depth_forward(plan, x, wg32, noise, w1, b1, w2, b2, logits, scores, idx, None if is_gshard else thr, stats,
-                              blob, y12[0], y12[1], y, ws, ev["fwd"] if ev else None)
+                              blob, estmm_plan, y12[0], y12[1], y, ws, ev["fwd"] if ev else None)
         config.routing_ = idx
         if any(ctx.needs_input_grad):
             ctx.owner = _BlobOwner(blob)
@@ -233,14 +234,15 @@ class FusedMoEDepth(torch.autograd.Function):
         ctx.param_dtypes = (wg.dtype, fc1_w.dtype, fc2_w.dtype, None if fc1_bias is None else fc1_bias.dtype,
                             None if fc2_bias is None else fc2_bias.dtype)
         ctx.dims = (T, top_k, E, d_in, hidden, d_out)
-        ctx.save_for_backward(x, wg32, w1, w2, state, idx, y12, blob)
+        ctx.save_for_backward(x, wg32, w1, w2, state, ints, y12, blob)
         ctx.set_materialize_grads(False)
         return y, stats[nstats - 1]
 
     @staticmethod
     def backward(ctx: Any, dy, dl_aux):
-        x, wg32, w1, w2, state, idx, y12, blob = ctx.saved_tensors
+        x, wg32, w1, w2, state, ints, y12, blob = ctx.saved_tensors
         T, top_k, E, d_in, hidden, d_out = ctx.dims
+        idx, estmm_plan = ints[:T * top_k].view(T, top_k), ints[T * top_k:]
         dev = x.device
         need_x, need_wg, need_w1, need_w2, need_b1, need_b2 = ctx.needs_input_grad[2:8]
         dt_wg, dt_w1, dt_w2, dt_b1, dt_b2 = ctx.param_dtypes
@@ -266,7 +268,7 @@ class FusedMoEDepth(torch.autograd.Function):
         thr, stats = state[2 * T * E:2 * T * E + T], state[2 * T * E + T:2 * T * E + T + nstats]
         ev = FusedMoEDepth.events
         ops.moe_depth_backward(ctx.plan, dy, g_aux, x, wg32, w1, w2, scores, idx, None if ctx.is_gshard else thr, stats,
-                               blob, y12[0], y12[1], dx, dwg, dw1, db1, dw2, db2, dy1, ws, ev["bwd"] if ev else None)
+                               blob, estmm_plan, y12[0], y12[1], dx, dwg, dw1, db1, dw2, db2, dy1, ws, ev["bwd"] if ev else None)
         ctx.owner = None
         ctx.config.stage = ctx.config.stage - 1
 

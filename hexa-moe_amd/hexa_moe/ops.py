@@ -446,25 +446,27 @@ def _event_array(events):
 
 
 def moe_depth_forward(plan, x, wg, noise, fc1_w, fc1_b, fc2_w, fc2_b, logits, scores, idx, thr, stats, route_blob,
-                      y1, y2, y, ws, events=None):
+                      estmm_plan, y1, y2, y, ws, events=None):
+    """estmm_plan: int32 [4E+1] that receives the work plan of the backward's ESTMM calls, or None."""
     import ctypes
     _dev(x, wg, noise, fc1_w, fc1_b, fc2_w, fc2_b, idx, route_blob, y1, y2, y, ws)
     ev, nev = _event_array(events)
     rc = _lib.load().hexa_moe_depth_forward(ctypes.byref(plan.desc), _ptr(x), _ptr(wg), _ptr(noise), _ptr(fc1_w),
                                             _ptr(fc1_b), _ptr(fc2_w), _ptr(fc2_b), _ptr(logits), _ptr(scores), _ptr(idx),
-                                            _ptr(thr), _ptr(stats), _ptr(route_blob), _ptr(y1), _ptr(y2), _ptr(y),
+                                            _ptr(thr), _ptr(stats), _ptr(route_blob), _ptr(estmm_plan), _ptr(y1), _ptr(y2), _ptr(y),
                                             _ptr(ws), ws.numel() * ws.element_size(), ev, nev, _stream())
     _lib.check(rc, "hexa_moe_depth_forward")
 
 
-def moe_depth_backward(plan, dy, grad_l_aux, x, wg, fc1_w, fc2_w, scores, idx, thr, stats, route_blob, y1, y2, dx, dwg,
-                       dw1, db1, dw2, db2, dy1, ws, events=None):
+def moe_depth_backward(plan, dy, grad_l_aux, x, wg, fc1_w, fc2_w, scores, idx, thr, stats, route_blob, estmm_plan, y1, y2,
+                       dx, dwg, dw1, db1, dw2, db2, dy1, ws, events=None):
+    """estmm_plan: the buffer moe_depth_forward filled for this routing, or None (the call then makes the plan)."""
     import ctypes
     _dev(dy, grad_l_aux, x, wg, fc1_w, fc2_w, route_blob, y1, y2, dx, dwg, dw1, db1, dw2, db2, dy1, ws)
     ev, nev = _event_array(events)
     rc = _lib.load().hexa_moe_depth_backward(ctypes.byref(plan.desc), _ptr(dy), _ptr(grad_l_aux), _ptr(x), _ptr(wg),
                                              _ptr(fc1_w), _ptr(fc2_w), _ptr(scores), _ptr(idx), _ptr(thr), _ptr(stats),
-                                             _ptr(route_blob), _ptr(y1), _ptr(y2), _ptr(dx), _ptr(dwg), _ptr(dw1),
+                                             _ptr(route_blob), _ptr(estmm_plan), _ptr(y1), _ptr(y2), _ptr(dx), _ptr(dwg), _ptr(dw1),
                                              _ptr(db1), _ptr(dw2), _ptr(db2), _ptr(dy1), _ptr(ws),
                                              ws.numel() * ws.element_size(), ev, nev, _stream())
     _lib.check(rc, "hexa_moe_depth_backward")

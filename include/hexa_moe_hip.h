@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define HEXA_ABI_VERSION 7
+#define HEXA_ABI_VERSION 8
 
 /* element types */
 #define HEXA_F32 0
@@ -295,33 +295,39 @@ int hexa_moe_depth_ws_bytes(const hexa_moe_depth_desc* d, int64_t* forward_bytes
  * stats / noise are ignored.
  * Then: route = hexa_route_build(idx); y1 = x.W1^T + b1 and y2 = gelu(y1) ([k][T][hidden], saved for the backward);
  * y [T][d_out] = sum over slots of y2.W2 + b2.  Biases may be NULL.
+ * plan (may be NULL): 4*num_experts+1 ints that receive the work plan of the backward's ESTMM calls (as
+ * hexa_estmm_plan; it depends on the routing only); hand the same buffer to hexa_moe_depth_backward and that call
+ * skips making it.  (With the GShard loss and up to 240 experts the router, the loss, the routing pass and the plan
+ * take three launches in all: the router counts its own tokens for the routing pass, whose scan launch finishes the
+ * loss and whose scatter launch makes the plan.)
  * events (may be NULL): 2*n caller-owned hipEvent_t handles; pair i is recorded on `stream` around major kernel i
  * (0: fc1 + GELU, 1: fc2 and its slot sum), for callers that time kernels inside a step; NULL handles in the
  * array are skipped. */
 int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* x, const float* wg, const float* noise,
                            const void* fc1_w, const void* fc1_b, const void* fc2_w, const void* fc2_b, float* logits,
-                           float* scores, int32_t* idx, float* thr, float* stats, int32_t* route, void* y1, void* y2,
-                           void* y, void* ws, int64_t ws_bytes, void* const* events, int num_events, void* stream);
+                           float* scores, int32_t* idx, float* thr, float* stats, int32_t* route, int32_t* plan, void* y1,
+                           void* y2, void* y, void* ws, int64_t ws_bytes, void* const* events, int num_events,
+                           void* stream);
 
 /* Backward of the same depth from dy [T][d_out] and (with wg) the device scalar grad_l_aux (NULL: the auxiliary
  * loss carries no gradient).  Results (each may be NULL to skip it): dx [T][d_in] = the expert path's input
  * gradient plus, with wg, the gate path's; dwg [E][d_in] fp32; dw1 [E][hidden][d_in], db1 [E][hidden],
  * dw2 [E][hidden][d_out], db2 [E][d_out].  dy1 is caller memory for the hidden gradient ([k][T][hidden] of act_dt);
- * its contents after the call are dy1 = (dy.W2^T) * gelu'(y1).
+ * its contents after the call are dy1 = (dy.W2^T) * gelu'(y1).  plan: the buffer the forward filled, or NULL.
  * events: pairs around (0) the dy1 kernel with its bias-gradient sums, (1) the dx kernel and its slot sum,
  * (2) ESTMM dW2, (3) ESTMM dW1. */
 int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void* dy, const float* grad_l_aux, const void* x,
                             const float* wg, const void* fc1_w, const void* fc2_w, const float* scores,
                             const int32_t* idx, const float* thr, const float* stats, const int32_t* route,
-                            const void* y1, const void* y2, void* dx, float* dwg, void* dw1, void* db1, void* dw2,
-                            void* db2, void* dy1, void* ws, int64_t ws_bytes, void* const* events, int num_events,
-                            void* stream);
+                            const int32_t* plan, const void* y1, const void* y2, void* dx, float* dwg, void* dw1,
+                            void* db1, void* dw2, void* db2, void* dy1, void* ws, int64_t ws_bytes, void* const* events,
+                            int num_events, void* stream);
 
 const char* hexa_last_error(void);
 int hexa_abi_version(void);
 
 /* Tuning / testing knobs of the kernels ("tile", "pipe", "general_kernels", "esmm_map", "esmm_group",
- * "estmm_group", "esmm_stream", "route_kernels", "ffn_fused"; 0 = automatic).  Each starts from an environment variable
+ * "estmm_group", "esmm_stream", "route_kernels", "batch", "ffn_fused"; 0 = automatic).  Each starts from an environment variable
  * (HEXA_MOE_TILE, HEXA_MOE_PIPE, HEXA_MOE_GENERAL_KERNELS, HEXA_ESMM_MAP, HEXA_ESMM_GROUP, HEXA_ESTMM_GROUP,
  * HEXA_ESMM_STREAM, HEXA_ROUTE_KERNELS).  Every setting computes the same results; the tests use it to run every kernel
  * variant.  No counterpart in the reference. */

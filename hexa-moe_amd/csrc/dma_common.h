@@ -231,10 +231,22 @@ template <typename TC> __device__ __forceinline__ float from_bits16(unsigned sho
     c.u = u;
     return (float)c.t;
 }
+// two floats rounded (to nearest even) into one 32-bit word, `a` in the low half: written as a two-element vector
+// conversion so that it becomes ONE instruction (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32) instead of two conversions,
+// a shift and an or -- the epilogues pack every element they produce
+template <typename TC> __device__ __forceinline__ unsigned pack2(float a, float b) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef TC tcx2_t __attribute__((ext_vector_type(2)));
+    f32x2_t v;
+    v.x = a; v.y = b;
+    union { tcx2_t t; unsigned u; } c;
+    c.t = __builtin_convertvector(v, tcx2_t);
+    return c.u;
+}
 template <typename TC> __device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
     uint2 o;
-    o.x = bits16<TC>(a) | ((unsigned)bits16<TC>(b) << 16);
-    o.y = bits16<TC>(c) | ((unsigned)bits16<TC>(d) << 16);
+    o.x = pack2<TC>(a, b);
+    o.y = pack2<TC>(c, d);
     return o;
 }
 

@@ -183,8 +183,7 @@ __global__ __launch_bounds__(FFN_NT, 4) void ffn16_fwd_kernel(FfnK p) {
                 unsigned vw[4] = {val[q].x, val[q].y, val[q].z, val[q].w}, aw[4];
 #pragma unroll
                 for (int u = 0; u < 4; ++u)   // applied to the value as stored (rounded), like act(y1) on the tensor
-                    aw[u] = bits16<TC>(gelu_fast(from_bits16<TC>(vw[u] & 0xffff))) |
-                            ((unsigned)bits16<TC>(gelu_fast(from_bits16<TC>(vw[u] >> 16))) << 16);
+                    aw[u] = pack2<TC>(gelu_fast(from_bits16<TC>(vw[u] & 0xffff)), gelu_fast(from_bits16<TC>(vw[u] >> 16)));
                 const uint4 act = make_uint4(aw[0], aw[1], aw[2], aw[3]);
                 if (tok >= 0) {
                     const size_t off = (hid_base + (size_t)tok * H) + h0 + c[q] * 8;

@@ -226,7 +226,7 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
                         for (int q = 0; q < 4; ++q) {
                             const float lo = from_bits16<TC>(vw[q] & 0xffff) * gelu_grad_fast(from_bits16<TC>(yw[q] & 0xffff));
                             const float hi = from_bits16<TC>(vw[q] >> 16) * gelu_grad_fast(from_bits16<TC>(yw[q] >> 16));
-                            vw[q] = bits16<TC>(lo) | ((unsigned)bits16<TC>(hi) << 16);
+                            vw[q] = pack2<TC>(lo, hi);
                         }
                         val = make_uint4(vw[0], vw[1], vw[2], vw[3]);
                     }
@@ -238,7 +238,7 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
                         for (int q = 0; q < 4; ++q) {
                             const float lo = from_bits16<TC>(vw[q] & 0xffff) + from_bits16<TC>(ow[q] & 0xffff);
                             const float hi = from_bits16<TC>(vw[q] >> 16) + from_bits16<TC>(ow[q] >> 16);
-                            vw[q] = bits16<TC>(lo) | ((unsigned)bits16<TC>(hi) << 16);
+                            vw[q] = pack2<TC>(lo, hi);
                         }
                         val = make_uint4(vw[0], vw[1], vw[2], vw[3]);
                     }
@@ -256,8 +256,7 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
                         unsigned vw[4] = {val.x, val.y, val.z, val.w};
 #pragma unroll
                         for (int q = 0; q < 4; ++q)
-                            vw[q] = bits16<TC>(gelu_fast(from_bits16<TC>(vw[q] & 0xffff))) |
-                                    ((unsigned)bits16<TC>(gelu_fast(from_bits16<TC>(vw[q] >> 16))) << 16);
+                            vw[q] = pack2<TC>(gelu_fast(from_bits16<TC>(vw[q] & 0xffff)), gelu_fast(from_bits16<TC>(vw[q] >> 16)));
                         store16(reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(p.out_act) + off),
                                 make_uint4(vw[0], vw[1], vw[2], vw[3]), p.stream_out == 1);
                     }

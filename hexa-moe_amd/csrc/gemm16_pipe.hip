@@ -87,9 +87,6 @@ __device__ __forceinline__ u32x4 global_load128_async(const void* p) {
 
 template <typename TC> __device__ __forceinline__ float lo16(unsigned w) { return from_bits16<TC>(w & 0xffff); }
 template <typename TC> __device__ __forceinline__ float hi16(unsigned w) { return from_bits16<TC>(w >> 16); }
-template <typename TC> __device__ __forceinline__ unsigned pack2(float a, float b) {
-    return bits16<TC>(a) | ((unsigned)bits16<TC>(b) << 16);
-}
 
 struct PipeK {
     EsmmK e;

@@ -584,10 +584,11 @@ int launch_estmm_dma_c(const EstmmArgs& a, hipStream_t st) {
     p.p_slot_rows = a.p_per_slot ? a.r.T : 0;
     p.q_slot_rows = a.q_per_slot ? a.r.T : 0;
     p.accumulate = a.accumulate;
-    // Runs of `group` tiles per XCD.  One row tile (with all its column tiles) per run is the fastest measured;
-    // 4 row tiles per run cut the launch's HBM fetch from 345 to 204 MB at the benchmark shape (the Q rows of an
-    // expert are then fetched by 3 of the 8 L2s instead of all of them) and cost 2 % in time.
-    p.group = p.ntn * std::max(1, option(OPT_ESTMM_GROUP));
+    // Runs of `group` tiles per XCD (workgroup ids go round-robin over the 8 XCDs, each with its own L2).  Runs of 3
+    // row tiles (with all their column tiles) cut the launch's HBM fetch at the benchmark shape from 340 to 230 MB
+    // (1.28x the operands: the Q rows of an expert are then fetched by fewer L2s) at the same time, 97 against 99 us;
+    // 4 fetch 202 MB and cost 3 %.  Results with few row tiles keep runs of one.
+    p.group = p.ntn * (option(OPT_ESTMM_GROUP) > 0 ? option(OPT_ESTMM_GROUP) : (p.mtn >= 6 ? 3 : 1));
     p.plan = nullptr; p.scratch = nullptr;
     int units = a.r.E;
     const int E = a.r.E;

@@ -24,6 +24,7 @@ for _p in (ROOT, os.path.join(ROOT, "hexa-moe_amd")):
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
 
 T, D, H, E, K_TOP = 18432, 384, 1536, 32, 2
 SEED = 1235
@@ -169,10 +170,24 @@ def main():
             kernels[label] = {"avg_us": round(avg_ms * 1e3, 2), "samples": len(vals), "bound": "mfma",
                               "tflops": round(tf, 1), "frac": round(tf / PEAK_BF16_TFLOPS, 4)}
         if ROOFLINE_KERNEL in kernels:
+            # fc1 + GELU per launch: 2*T*k*d*h FLOP; algorithmic bytes = x rows once (T*d), W1 and b1 once, y1 and y2
+            # written once (2 * T*k*h), 2-byte elements.  Its arithmetic intensity (156 FLOP/B) is below the machine's
+            # ridge (2.5 PFLOP/s / 8 TB/s = 312 FLOP/B): the roof that bounds it is HBM, at 0.5 of the MFMA peak.
             d = kernels[ROOFLINE_KERNEL]
-            roofline = {"kernel": ROOFLINE_KERNEL, "bound": "mfma", "achieved": d["tflops"], "peak": PEAK_BF16_TFLOPS,
-                        "unit": "TFLOP/s", "frac": d["frac"], "traffic": measured_traffic(ROOFLINE_KERNEL),
-                        "algorithmic_flop": gemm, "avg_us": d["avg_us"]}
+            alg_bytes = 2.0 * (T * D + E * H * D + E * H + 2 * T * K_TOP * H)
+            secs = d["avg_us"] * 1e-6
+            gbs = alg_bytes / secs / 1e9
+            intensity, ridge = gemm / alg_bytes, PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
+            hbm_bound = intensity < ridge
+            roofline = {"kernel": ROOFLINE_KERNEL, "bound": "hbm" if hbm_bound else "mfma",
+                        "achieved": round(gbs, 1) if hbm_bound else d["tflops"],
+                        "peak": PEAK_HBM_GBS if hbm_bound else PEAK_BF16_TFLOPS,
+                        "unit": "GB/s" if hbm_bound else "TFLOP/s",
+                        "frac": round(gbs / PEAK_HBM_GBS, 4) if hbm_bound else d["frac"],
+                        "traffic": measured_traffic(ROOFLINE_KERNEL),
+                        "algorithmic_bytes": alg_bytes, "algorithmic_flop": gemm, "avg_us": d["avg_us"],
+                        "arithmetic_intensity_flop_per_byte": round(intensity, 1), "ridge_flop_per_byte": round(ridge, 1),
+                        "hbm_frac": round(gbs / PEAK_HBM_GBS, 4), "mfma_tflops": d["tflops"], "mfma_frac": d["frac"]}
 
     # ---- CPU baseline: the oracle's plain-PyTorch fp32 evaluation of the same layer on the host ----
     cpu = None

@@ -26,6 +26,7 @@ OptEntry g_opts[OPT_COUNT] = {
     {"esmm_stream", "HEXA_ESMM_STREAM", 0, false}, {"route_kernels", "HEXA_ROUTE_KERNELS", 0, false},
     {"batch", "HEXA_MOE_BATCH", 0, false},
     {"ffn_fused", "HEXA_MOE_FFN_FUSED", 0, false},
+    {"gate_router", "HEXA_MOE_GATE_ROUTER", 0, false},
 };
 }  // namespace
 

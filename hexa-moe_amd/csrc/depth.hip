@@ -150,12 +150,19 @@ extern "C" int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* 
     bool routed = false;
     if (wg) {
         if (!logits || !scores || !stats || (d->loss == 1 && !thr)) HEXA_FAIL(HEXA_ERR_ARG, "%s: null router state", who);
-        RUN(hexa_gate_logits(logits, x, wg, T, d->d_in, E, d->act_dt, stream));
-        if (d->loss == 0 && router_hist_supported(E)) {
-            // three launches for router, loss, routing pass and plan: the router counts its own tokens for the routing
-            // pass, whose scan launch carries the loss and whose scatter launch carries the plan
+        const bool front3 = d->loss == 0 && router_hist_supported(E);
+        const bool one_launch = front3 && option(OPT_GATE_ROUTER) != 2 && T > 0 && gate_router_supported(d->d_in, E, d->act_dt);
+        if (!one_launch) RUN(hexa_gate_logits(logits, x, wg, T, d->d_in, E, d->act_dt, stream));
+        if (front3) {
+            // three launches for gate, router, loss, routing pass and plan: the gate's logits go straight into the
+            // router's tile (two launches above GATE_ROUTER_MAX_E experts), the router counts its own tokens for the
+            // routing pass, whose scan launch carries the loss and whose scatter launch carries the plan
             RUN(router_forward_check(T, E, k, true));
-            RUN(launch_router_fwd(scores, idx, logits, noise, d->noise_scale, T, E, k, w.router, w.hist, (hipStream_t)stream));
+            if (one_launch)
+                RUN(launch_gate_router(logits, scores, idx, x, wg, noise, d->noise_scale, T, d->d_in, E, k, d->act_dt, w.router,
+                                       w.hist, (hipStream_t)stream));
+            else
+                RUN(launch_router_fwd(scores, idx, logits, noise, d->noise_scale, T, E, k, w.router, w.hist, (hipStream_t)stream));
             RUN(launch_route_from_hist(idx, T, k, E, route, w.hist, router_tokens_per_workgroup(), stats + 2 * E, stats,
                                        stats + E, w.router, plan, plan_slots, (hipStream_t)stream));
             routed = true;

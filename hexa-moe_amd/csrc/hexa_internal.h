@@ -96,6 +96,7 @@ enum Opt {
     OPT_ROUTE_KERNELS,  // HEXA_ROUTE_KERNELS: 3 = always the three-launch routing pass, 1 = one launch up to 65536 tokens
     OPT_BATCH,          // HEXA_MOE_BATCH: 2 = every small kernel of the depth backward in a launch of its own
     OPT_FFN_FUSED,      // HEXA_MOE_FFN_FUSED: 1 = hexa_moe_depth_forward runs fc1, GELU and fc2 in one kernel where it is covered
+    OPT_GATE_ROUTER,    // HEXA_MOE_GATE_ROUTER: 2 = hexa_moe_depth_forward runs the gate projection and the router as two launches
     OPT_COUNT
 };
 int option(int id);
@@ -126,6 +127,9 @@ int router_tokens_per_workgroup();
 int router_forward_check(int T, int E, int k, bool ptrs_ok);
 int launch_router_fwd(float* scores, int32_t* idx, const float* logits, const float* noise, float noise_scale, int T, int E,
                       int k, float* ws, int32_t* hist, hipStream_t st);
+bool gate_router_supported(int d, int E, int x_dt);
+int launch_gate_router(float* logits, float* scores, int32_t* idx, const void* x, const float* wg, const float* noise,
+                       float noise_scale, int T, int d, int E, int k, int x_dt, float* ws, int32_t* hist, hipStream_t st);
 int launch_route_from_hist(const int32_t* idx, int T, int k, int E, int32_t* route, int32_t* hist, int unit_tokens,
                            float* l_aux, float* me, float* ce, const float* router_ws, int32_t* plan, int plan_slots,
                            hipStream_t st);

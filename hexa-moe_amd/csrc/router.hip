@@ -8,6 +8,7 @@
 //            hexa_moe_cuda/hexa_moe/impls/layers.py:476-484 (top-k), impls/losses.py:12-19 (GShard loss).
 #include "hexa_internal.h"
 #include "small_bodies.h"
+#include "gate_bodies.h"
 
 namespace hexa {
 namespace {
@@ -102,108 +103,97 @@ __host__ __device__ constexpr int router_pitch(int E) {
 
 // hist (optional): [k][workgroups][E] ints, per slot the number of this workgroup's 64 tokens that chose each expert
 // -- the histogram the routing pass starts from (units of 64 tokens), so that pass needs no counting launch.
-__global__ __launch_bounds__(ROUTER_TB * ROUTER_G) void router_fwd4_kernel(
-    float* __restrict__ scores, int32_t* __restrict__ idx, float* __restrict__ part_me, float* __restrict__ part_cnt,
-    const float* __restrict__ logits, const float* __restrict__ noise, float noise_scale, int num_tokens, int E, int k,
-    int32_t* __restrict__ hist) {
-    extern __shared__ float sh[];          // cnt[E], the tile [64][P], then hist[k][E]
-    float* s_cnt = sh;
-    const int P = router_pitch(E);
-    float* tile = sh + ((E + 3) & ~3);
-    int* s_hist = reinterpret_cast<int*>(tile + ROUTER_TB * P);
+// LDS of the four-lanes-per-token router: cnt[E], the tile [64][P], then hist[k][E]
+struct Router4Lds {
+    float* cnt; float* tile; int* hist; int P;
+    __device__ __forceinline__ Router4Lds(float* sh, int E) : cnt(sh), tile(sh + ((E + 3) & ~3)), P(router_pitch(E)) {
+        hist = reinterpret_cast<int*>(tile + ROUTER_TB * P);
+    }
+};
+__host__ __device__ constexpr size_t router4_lds_floats(int E, int k, bool hist) {
+    return (size_t)((E + 3) & ~3) + (size_t)ROUTER_TB * router_pitch(E) + (hist ? (size_t)k * E : 0);
+}
+
+// Everything behind the tile of (noisy) logits: softmax, top-k, loss partials, histogram, scores out.  The tile
+// holds rows [t0, t0 + rows) of the workgroup; the counters have been cleared; a barrier separates both from here.
+// The workgroup has at least ROUTER_TB * ROUTER_G threads.
+__device__ __forceinline__ void router4_body(const Router4Lds& L, float* __restrict__ scores, int32_t* __restrict__ idx,
+                                             float* __restrict__ part_me, float* __restrict__ part_cnt,
+                                             int32_t* __restrict__ hist, int t0, int rows, int E, int k) {
+    float* s_cnt = L.cnt;
+    float* tile = L.tile;
+    int* s_hist = L.hist;
+    const int P = L.P;
     const int tid = threadIdx.x;
-    const int t0 = blockIdx.x * ROUTER_TB;
-    const int rows = min(ROUTER_TB, num_tokens - t0);
-    for (int i = tid; i < E; i += blockDim.x) s_cnt[i] = 0.f;
-    if (hist)
-        for (int i = tid; i < k * E; i += blockDim.x) s_hist[i] = 0;
-    // ---- tile in: element i of the contiguous block [rows][E] ----
     const size_t g0 = (size_t)t0 * E;
     const int total = rows * E;
-    if ((E & 3) == 0) {
-        for (int i = tid * 4; i < total; i += blockDim.x * 4) {
-            float4 v = *reinterpret_cast<const float4*>(logits + g0 + i);
-            if (noise) {
-                const float4 n = *reinterpret_cast<const float4*>(noise + g0 + i);
-                v.x += noise_scale * n.x; v.y += noise_scale * n.y; v.z += noise_scale * n.z; v.w += noise_scale * n.w;
+    if (tid < ROUTER_TB * ROUTER_G) {   // four lanes per token; further wavefronts of the workgroup help with the sums only
+        const int r = tid >> 2, q = tid & 3;
+        const int t = t0 + r;
+        const bool ok = r < rows;
+        float* row = tile + r * P;
+        // The selection is total: a row of NaN scores (NaN or +Inf logits) beats no entry, so the lists start out as
+        // the lanes' own experts in index order and such a token ends up with experts 0..k-1 (torch.topk also returns
+        // valid ids for NaN rows); its NaN then reaches the output through the token's own features and the loss
+        // through the score sums.
+        float bv[MAX_TOPK];
+        int bi[MAX_TOPK];
+    #pragma unroll
+        for (int j = 0; j < MAX_TOPK; ++j) { bv[j] = -INFINITY; bi[j] = q + ROUTER_G * j; }
+        if (ok) {
+            float mx = -INFINITY;
+            for (int e = q; e < E; e += ROUTER_G) mx = fmaxf(mx, row[e]);
+            mx = fmaxf(mx, __shfl_xor(mx, 1));
+            mx = fmaxf(mx, __shfl_xor(mx, 2));
+            float sum = 0.f;
+            for (int e = q; e < E; e += ROUTER_G) {
+                const float ex = expf(row[e] - mx);
+                row[e] = ex;
+                sum += ex;
             }
-            const int r = i / E, e = i - r * E;
-            *reinterpret_cast<float4*>(tile + r * P + e) = v;
-        }
-    } else {
-        for (int i = tid; i < total; i += blockDim.x) {
-            float v = logits[g0 + i];
-            if (noise) v += noise_scale * noise[g0 + i];
-            const int r = i / E, e = i - r * E;
-            tile[r * P + e] = v;
-        }
-    }
-    __syncthreads();
-    const int r = tid >> 2, q = tid & 3;
-    const int t = t0 + r;
-    const bool ok = r < rows;
-    float* row = tile + r * P;
-    // The selection is total: a row of NaN scores (NaN or +Inf logits) beats no entry, so the lists start out as
-    // the lanes' own experts in index order and such a token ends up with experts 0..k-1 (torch.topk also returns
-    // valid ids for NaN rows); its NaN then reaches the output through the token's own features and the loss
-    // through the score sums.
-    float bv[MAX_TOPK];
-    int bi[MAX_TOPK];
-#pragma unroll
-    for (int j = 0; j < MAX_TOPK; ++j) { bv[j] = -INFINITY; bi[j] = q + ROUTER_G * j; }
-    if (ok) {
-        float mx = -INFINITY;
-        for (int e = q; e < E; e += ROUTER_G) mx = fmaxf(mx, row[e]);
-        mx = fmaxf(mx, __shfl_xor(mx, 1));
-        mx = fmaxf(mx, __shfl_xor(mx, 2));
-        float sum = 0.f;
-        for (int e = q; e < E; e += ROUTER_G) {
-            const float ex = expf(row[e] - mx);
-            row[e] = ex;
-            sum += ex;
-        }
-        sum += __shfl_xor(sum, 1);         // (s0 + s1) + (s2 + s3) on every lane of the quad
-        sum += __shfl_xor(sum, 2);
-        const float inv = 1.0f / sum;
-        for (int e = q; e < E; e += ROUTER_G) {
-            const float sc = row[e] * inv;
-            row[e] = sc;
-            topk_insert(bv, bi, k, sc, e);  // ascending e, strict '>': the lower index stays ahead on ties
-        }
-    } else {
-        for (int e = q; e < E; e += ROUTER_G) row[e] = 0.f;
-    }
-    // merge the four lists: k rounds, each takes the best head (greater score; lower index on ties)
-    int pick[MAX_TOPK];
-#pragma unroll
-    for (int j = 0; j < MAX_TOPK; ++j) {
-        pick[j] = 0;
-        if (j < k) {
-            float hv = bv[0];
-            int hi = bi[0];
-#pragma unroll
-            for (int m = 1; m <= 2; m <<= 1) {
-                const float ov = __shfl_xor(hv, m);
-                const int oi = __shfl_xor(hi, m);
-                if (ov > hv || (ov == hv && oi < hi)) { hv = ov; hi = oi; }
+            sum += __shfl_xor(sum, 1);         // (s0 + s1) + (s2 + s3) on every lane of the quad
+            sum += __shfl_xor(sum, 2);
+            const float inv = 1.0f / sum;
+            for (int e = q; e < E; e += ROUTER_G) {
+                const float sc = row[e] * inv;
+                row[e] = sc;
+                topk_insert(bv, bi, k, sc, e);  // ascending e, strict '>': the lower index stays ahead on ties
             }
-            pick[j] = hi;
-            if (hi == bi[0]) {
-#pragma unroll
-                for (int m = 0; m + 1 < MAX_TOPK; ++m) { bv[m] = bv[m + 1]; bi[m] = bi[m + 1]; }
-                bv[MAX_TOPK - 1] = -INFINITY;
-                bi[MAX_TOPK - 1] = 0x7fffffff;
+        } else {
+            for (int e = q; e < E; e += ROUTER_G) row[e] = 0.f;
+        }
+        // merge the four lists: k rounds, each takes the best head (greater score; lower index on ties)
+        int pick[MAX_TOPK];
+    #pragma unroll
+        for (int j = 0; j < MAX_TOPK; ++j) {
+            pick[j] = 0;
+            if (j < k) {
+                float hv = bv[0];
+                int hi = bi[0];
+    #pragma unroll
+                for (int m = 1; m <= 2; m <<= 1) {
+                    const float ov = __shfl_xor(hv, m);
+                    const int oi = __shfl_xor(hi, m);
+                    if (ov > hv || (ov == hv && oi < hi)) { hv = ov; hi = oi; }
+                }
+                pick[j] = hi;
+                if (hi == bi[0]) {
+    #pragma unroll
+                    for (int m = 0; m + 1 < MAX_TOPK; ++m) { bv[m] = bv[m + 1]; bi[m] = bi[m + 1]; }
+                    bv[MAX_TOPK - 1] = -INFINITY;
+                    bi[MAX_TOPK - 1] = 0x7fffffff;
+                }
             }
         }
-    }
-    if (ok) {
-#pragma unroll
-        for (int j = 0; j < MAX_TOPK; ++j)
-            if (j < k && (j & 3) == q) {
-                idx[(size_t)t * k + j] = pick[j];
-                if (hist) atomicAdd(&s_hist[j * E + pick[j]], 1);
-            }
-        if (q == 0) atomicAdd(&s_cnt[pick[0]], 1.0f);   // exact: at most 64 ones per counter
+        if (ok) {
+    #pragma unroll
+            for (int j = 0; j < MAX_TOPK; ++j)
+                if (j < k && (j & 3) == q) {
+                    idx[(size_t)t * k + j] = pick[j];
+                    if (hist) atomicAdd(&s_hist[j * E + pick[j]], 1);
+                }
+            if (q == 0) atomicAdd(&s_cnt[pick[0]], 1.0f);   // exact: at most 64 ones per counter
+        }
     }
     __syncthreads();
     // per-expert sums over the 64 tokens, in token order; the scores leave coalesced
@@ -230,6 +220,135 @@ __global__ __launch_bounds__(ROUTER_TB * ROUTER_G) void router_fwd4_kernel(
             scores[g0 + i] = tile[rr * P + e];
         }
     }
+}
+
+__global__ __launch_bounds__(ROUTER_TB * ROUTER_G) void router_fwd4_kernel(
+    float* __restrict__ scores, int32_t* __restrict__ idx, float* __restrict__ part_me, float* __restrict__ part_cnt,
+    const float* __restrict__ logits, const float* __restrict__ noise, float noise_scale, int num_tokens, int E, int k,
+    int32_t* __restrict__ hist) {
+    extern __shared__ float sh[];
+    const Router4Lds L(sh, E);
+    const int P = L.P;
+    float* tile = L.tile;
+    const int tid = threadIdx.x;
+    const int t0 = blockIdx.x * ROUTER_TB;
+    const int rows = min(ROUTER_TB, num_tokens - t0);
+    for (int i = tid; i < E; i += blockDim.x) L.cnt[i] = 0.f;
+    if (hist)
+        for (int i = tid; i < k * E; i += blockDim.x) L.hist[i] = 0;
+    // ---- tile in: element i of the contiguous block [rows][E] ----
+    const size_t g0 = (size_t)t0 * E;
+    const int total = rows * E;
+    if ((E & 3) == 0) {
+        for (int i = tid * 4; i < total; i += blockDim.x * 4) {
+            float4 v = *reinterpret_cast<const float4*>(logits + g0 + i);
+            if (noise) {
+                const float4 n = *reinterpret_cast<const float4*>(noise + g0 + i);
+                v.x += noise_scale * n.x; v.y += noise_scale * n.y; v.z += noise_scale * n.z; v.w += noise_scale * n.w;
+            }
+            const int r = i / E, e = i - r * E;
+            *reinterpret_cast<float4*>(tile + r * P + e) = v;
+        }
+    } else {
+        for (int i = tid; i < total; i += blockDim.x) {
+            float v = logits[g0 + i];
+            if (noise) v += noise_scale * noise[g0 + i];
+            const int r = i / E, e = i - r * E;
+            tile[r * P + e] = v;
+        }
+    }
+    __syncthreads();
+    router4_body(L, scores, idx, part_me, part_cnt, hist, t0, rows, E, k);
+}
+
+// The gate's projection and the router in one launch for 16-bit or fp32 token tensors and up to GATE_ROUTER_MAX_E
+// experts: the workgroup's 64 x E logits go from the matrix cores into the router's LDS tile (and out to `logits`,
+// which the backward reads) instead of through a launch boundary.  The arithmetic is that of gate_fwd_kernel, sum
+// for sum: a 32-token block's model dimension is cut into the same four quarters, one per wavefront, each
+// accumulated by the same sequence of products and added in the same order, so the logits are bit-identical to
+// hexa_gate_logits'.  Eight wavefronts (two token blocks) project; the first four then route.
+constexpr int GATE_ROUTER_MAX_E = 64;
+constexpr int GATE_ROUTER_NT = 2 * ROUTER_TB * ROUTER_G;
+template <typename T>
+__global__ __launch_bounds__(GATE_ROUTER_NT) void gate_router_kernel(
+    float* __restrict__ logits, float* __restrict__ scores, int32_t* __restrict__ idx, float* __restrict__ part_me,
+    float* __restrict__ part_cnt, const T* __restrict__ x, const float* __restrict__ wg, const float* __restrict__ noise,
+    float noise_scale, int num_tokens, int d, int E, int k, int32_t* __restrict__ hist) {
+    extern __shared__ float sh[];
+    __shared__ float part[2][4][16][64];             // [token block][quarter of d][result register][lane]
+    const Router4Lds L(sh, E);
+    const int P = L.P;
+    float* tile = L.tile;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int t0 = blockIdx.x * ROUTER_TB;
+    const int rows = min(ROUTER_TB, num_tokens - t0);
+    for (int i = tid; i < E; i += blockDim.x) L.cnt[i] = 0.f;
+    if (hist)
+        for (int i = tid; i < k * E; i += blockDim.x) L.hist[i] = 0;
+    // ---- the gate: logits of 64 tokens into the tile ----
+    const int r = lane & 31, h = lane >> 5;
+    const int blk = wave >> 2, quarter = wave & 3;
+    const int pieces = d >> 3;                       // 8 contraction indices per piece
+    const int chunks = (pieces + 1) >> 1;            // a chunk = one piece per half-wavefront
+    const int c0 = (chunks * quarter) >> 2, c1 = (chunks * (quarter + 1)) >> 2;
+    const bool tok_ok = t0 + 32 * blk + r < num_tokens;
+    const T* xrow = x + (size_t)(tok_ok ? t0 + 32 * blk + r : 0) * d;
+    for (int e0 = 0; e0 < E; e0 += 32) {
+        const bool exp_ok = e0 + r < E;
+        const float* wrow = wg + (size_t)(exp_ok ? e0 + r : 0) * d;
+        f32x16 acc = zero16();
+        for (int c = c0; c < c1; c += FWD_NB) {
+            float xv[FWD_NB][8], wv[FWD_NB][8];
+#pragma unroll
+            for (int u = 0; u < FWD_NB; ++u) {
+                const int piece = 2 * (c + u) + h;
+                const bool ok = c + u < c1 && piece < pieces;
+                LoadN<T, 8>::run(xrow + (ok ? piece : 0) * 8, ok && tok_ok, xv[u]);
+                LoadN<float, 8>::run(wrow + (ok ? piece : 0) * 8, ok && exp_ok, wv[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < FWD_NB; ++u)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[u][i], wv[u][i], acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) part[blk][quarter][v][lane] = acc[v];
+        __syncthreads();
+        // wavefront (blk, w) finishes result registers 4w .. 4w+3: token row 8w + 4h + q of the block, expert column r
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int v = 4 * quarter + q;
+            const float sum = ((part[blk][0][v][lane] + part[blk][1][v][lane]) + part[blk][2][v][lane]) + part[blk][3][v][lane];
+            const int row = 32 * blk + 8 * quarter + 4 * h + q;
+            if (exp_ok) tile[row * P + e0 + r] = sum;
+        }
+        __syncthreads();   // the partial sums have been consumed (the next expert block overwrites them)
+    }
+    // ---- the logits leave as they are; the noise joins the tile only ----
+    const size_t g0 = (size_t)t0 * E;
+    const int total = rows * E;
+    if ((E & 3) == 0) {
+        for (int i = tid * 4; i < total; i += blockDim.x * 4) {
+            const int rr = i / E, e = i - rr * E;
+            float4 v = *reinterpret_cast<const float4*>(tile + rr * P + e);
+            *reinterpret_cast<float4*>(logits + g0 + i) = v;
+            if (noise) {
+                const float4 n = *reinterpret_cast<const float4*>(noise + g0 + i);
+                v.x += noise_scale * n.x; v.y += noise_scale * n.y; v.z += noise_scale * n.z; v.w += noise_scale * n.w;
+                *reinterpret_cast<float4*>(tile + rr * P + e) = v;
+            }
+        }
+    } else {
+        for (int i = tid; i < total; i += blockDim.x) {
+            const int rr = i / E, e = i - rr * E;
+            const float v = tile[rr * P + e];
+            logits[g0 + i] = v;
+            if (noise) tile[rr * P + e] = v + noise_scale * noise[g0 + i];
+        }
+    }
+    __syncthreads();
+    router4_body(L, scores, idx, part_me, part_cnt, hist, t0, rows, E, k);
 }
 
 // The GShard loss from the workgroup partials (see small_bodies.h) as a launch of its own.
@@ -446,13 +565,37 @@ int launch_router_fwd(float* scores, int32_t* idx, const float* logits, const fl
     float* part_me = ws;
     float* part_cnt = ws + (size_t)nb * E;
     if (E <= ROUTER_LDS_E)
-        hipLaunchKernelGGL(router_fwd4_kernel, dim3(nb), dim3(ROUTER_TB * ROUTER_G),
-                           sizeof(float) * (((E + 3) & ~3) + ROUTER_TB * router_pitch(E) + (hist ? k * E : 0)), st, scores, idx,
-                           part_me, part_cnt, logits, noise, noise_scale, T, E, k, hist);
+        hipLaunchKernelGGL(router_fwd4_kernel, dim3(nb), dim3(ROUTER_TB * ROUTER_G), sizeof(float) * router4_lds_floats(E, k, hist != nullptr),
+                           st, scores, idx, part_me, part_cnt, logits, noise, noise_scale, T, E, k, hist);
     else
         hipLaunchKernelGGL(router_fwd_kernel, dim3(nb), dim3(ROUTER_TB), sizeof(float) * 2 * E, st, scores, idx,
                            part_me, part_cnt, logits, noise, noise_scale, T, E, k);
     HEXA_CHECK_LAUNCH("router_fwd");
+    return HEXA_OK;
+}
+
+// gate projection + router in one launch (see gate_router_kernel); same results as hexa_gate_logits followed by
+// launch_router_fwd
+bool gate_router_supported(int d, int E, int x_dt) {
+    return E <= GATE_ROUTER_MAX_E && (d % 8) == 0 && (x_dt == HEXA_F32 || x_dt == HEXA_BF16 || x_dt == HEXA_F16);
+}
+int launch_gate_router(float* logits, float* scores, int32_t* idx, const void* x, const float* wg, const float* noise,
+                       float noise_scale, int T, int d, int E, int k, int x_dt, float* ws, int32_t* hist, hipStream_t st) {
+    const int nb = div_up(T, ROUTER_TB);
+    float* part_me = ws;
+    float* part_cnt = ws + (size_t)nb * E;
+    const size_t lds = sizeof(float) * router4_lds_floats(E, k, hist != nullptr);
+    const dim3 grid(nb), block(GATE_ROUTER_NT);
+    if (x_dt == HEXA_F32)
+        hipLaunchKernelGGL(gate_router_kernel<float>, grid, block, lds, st, logits, scores, idx, part_me, part_cnt, (const float*)x, wg,
+                           noise, noise_scale, T, d, E, k, hist);
+    else if (x_dt == HEXA_BF16)
+        hipLaunchKernelGGL(gate_router_kernel<__bf16>, grid, block, lds, st, logits, scores, idx, part_me, part_cnt, (const __bf16*)x, wg,
+                           noise, noise_scale, T, d, E, k, hist);
+    else
+        hipLaunchKernelGGL(gate_router_kernel<_Float16>, grid, block, lds, st, logits, scores, idx, part_me, part_cnt,
+                           (const _Float16*)x, wg, noise, noise_scale, T, d, E, k, hist);
+    HEXA_CHECK_LAUNCH("gate_router");
     return HEXA_OK;
 }
 }  // namespace hexa

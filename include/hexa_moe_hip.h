@@ -327,7 +327,7 @@ const char* hexa_last_error(void);
 int hexa_abi_version(void);
 
 /* Tuning / testing knobs of the kernels ("tile", "pipe", "general_kernels", "esmm_map", "esmm_group",
- * "estmm_group", "esmm_stream", "route_kernels", "batch", "ffn_fused"; 0 = automatic).  Each starts from an environment variable
+ * "estmm_group", "esmm_stream", "route_kernels", "batch", "ffn_fused", "gate_router"; 0 = automatic).  Each starts from an environment variable
  * (HEXA_MOE_TILE, HEXA_MOE_PIPE, HEXA_MOE_GENERAL_KERNELS, HEXA_ESMM_MAP, HEXA_ESMM_GROUP, HEXA_ESTMM_GROUP,
  * HEXA_ESMM_STREAM, HEXA_ROUTE_KERNELS).  Every setting computes the same results; the tests use it to run every kernel
  * variant.  No counterpart in the reference. */

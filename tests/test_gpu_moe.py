@@ -310,3 +310,42 @@ def test_one_kernel_ffn_forward(dev, dtype, T, d, E, k, bias):
     assert_close(dxa, dxb, TOL[dtype] / 4, "dx")
     for u, v in zip(ga, gb):
         assert_close(u, v, TOL[dtype] / 4, "parameter gradient")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,d,E,k,train", [(2500, 256, 16, 2, True), (2300, 384, 32, 2, False), (1900, 128, 5, 3, True),
+                                           (130, 264, 33, 2, True), (63, 8, 64, 1, False), (4097, 96, 7, 4, True)])
+def test_gate_and_router_in_one_launch(dev, dtype, T, d, E, k, train):
+    """The depth call's front end with the gate projection and the router in one kernel (the default up to 64
+    experts) against the same call with the two as separate launches (library option "gate_router" = 2): the one
+    kernel repeats the gate's sums in the same order, so routing, y, l_aux and every gradient are identical -- with
+    gate noise (train mode, same seed), expert counts that are no multiple of 4 or span two 32-expert blocks, and a
+    last workgroup with fewer than 64 tokens."""
+    from hexa_moe import _lib
+    lib = _lib.load()
+    m = _module([d], [0], E=E, k=k, act=F.gelu, noise=1.0).to(dev).to(dtype)
+    m.train(train)
+    m.gates[0].wg.weight.data = m.gates[0].wg.weight.data.float()
+    m.fused_depth = True
+    g = torch.Generator().manual_seed(29)
+    x = torch.randn(T, d, generator=g).to(dtype).to(dev)
+    dy = torch.randn(T, d, generator=g).to(dtype).to(dev)
+    res = []
+    try:
+        for separate in (0, 2):
+            _lib.check(lib.hexa_set_option(b"gate_router", separate), "hexa_set_option")
+            torch.manual_seed(5)                      # the gate noise of both runs
+            m.zero_grad(set_to_none=True)
+            xi = x.clone().requires_grad_(True)
+            y, l_aux = m(0, xi)
+            torch.autograd.backward([y, l_aux], [dy, torch.full((), 2.0, device=dev)])
+            torch.cuda.synchronize()
+            res.append((m.dispatch_params.routing_.clone(), y.detach().clone(), l_aux.detach().clone(), xi.grad.clone(),
+                        [p.grad.clone() for p in m.parameters() if p.grad is not None]))
+    finally:
+        _lib.check(lib.hexa_set_option(b"gate_router", 0), "hexa_set_option")
+    (ra, ya, la, dxa, ga), (rb, yb, lb, dxb, gb) = res
+    assert torch.equal(ra, rb) and torch.equal(ya, yb) and torch.equal(la, lb) and torch.equal(dxa, dxb)
+    assert len(ga) == len(gb) and len(ga) >= 3
+    for u, v in zip(ga, gb):
+        assert torch.equal(u, v)

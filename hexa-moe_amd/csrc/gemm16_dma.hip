@@ -80,17 +80,23 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
     if (tid < BM) sTok[tid] = tid < rows ? p.token_ids[(size_t)s * p.T + row_start + tid] : -1;
     __syncthreads();
 
-    // ---- source pointers of this lane's copies ----
-    const char* zero = reinterpret_cast<const char*>(g_zero_block);
-    const char* srcR[C::R_CPW]; int stepR[C::R_CPW];
-    const char* srcF[C::F_CPW]; int stepF[C::F_CPW];
+    // ---- sources of this lane's copies: a base every lane shares plus a 32-bit byte offset per lane ----
+    // (the copy instruction then reads ONE address register per lane and a scalar pair instead of two registers per
+    // lane: next to wavefronts that issue MFMAs back to back, a CU moves 28 B/clk with this form against 10 with
+    // 64-bit lane addresses, and the MFMAs themselves run at 80 % instead of 60 % -- the launcher keeps tensors of
+    // 4 GiB and more off this kernel).  Lanes that have nothing to fetch (rows past the end of a segment, columns
+    // past N) re-read the first bytes of the tensor: what they produce is never stored.
+    const char* const xbase = reinterpret_cast<const char*>(p.x);
+    const char* const wbase = reinterpret_cast<const char*>(p.w) + (size_t)e * K * N * 2;
+    unsigned offR[C::R_CPW]; int stepR[C::R_CPW];
+    unsigned offF[C::F_CPW]; int stepF[C::F_CPW];
 #pragma unroll
     for (int i = 0; i < C::R_CPW; ++i) {   // token rows, KC
         int row, kc;
         kc_lane<BK>(wave + NW * i, lane, row, kc);
         const int tok = sTok[row];
         const bool ok = tok >= 0;
-        srcR[i] = ok ? reinterpret_cast<const char*>(p.x) + (((size_t)p.x_slot_rows * s + tok) * K + kc * 8) * 2 : zero;
+        offR[i] = ok ? (unsigned)((((size_t)p.x_slot_rows * s + tok) * K + kc * 8) * 2) : 0u;
         stepR[i] = ok ? BK * 2 : 0;
     }
 #pragma unroll
@@ -100,14 +106,14 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
             ks_lane<BN>(wave + NW * i, lane, kk, ch);
             const int n = n0 + ch * 8;
             const bool ok = n < N;
-            srcF[i] = ok ? reinterpret_cast<const char*>(p.w) + (((size_t)e * K + kk) * N + n) * 2 : zero;
+            offF[i] = ok ? (unsigned)(((size_t)kk * N + n) * 2) : 0u;
             stepF[i] = ok ? BK * N * 2 : 0;
         } else {         // w[e][n][k], KC
             int row, kc;
             kc_lane<BK>(wave + NW * i, lane, row, kc);
             const int n = n0 + row;
             const bool ok = n < N;
-            srcF[i] = ok ? reinterpret_cast<const char*>(p.w) + (((size_t)e * N + n) * K + kc * 8) * 2 : zero;
+            offF[i] = ok ? (unsigned)(((size_t)n * K + kc * 8) * 2) : 0u;
             stepF[i] = ok ? BK * 2 : 0;
         }
     }
@@ -115,13 +121,13 @@ __global__ __launch_bounds__(C::NT, C::MINW) void esmm16_dma_kernel(EsmmK p) {
         char* base = smem + stage * C::STAGE_BYTES;
 #pragma unroll
         for (int i = 0; i < C::R_CPW; ++i) {
-            dma16(srcR[i], base + (wave + NW * i) * 1024);
-            srcR[i] += stepR[i];
+            dma16(xbase + (size_t)offR[i], base + (wave + NW * i) * 1024);
+            offR[i] += stepR[i];
         }
 #pragma unroll
         for (int i = 0; i < C::F_CPW; ++i) {
-            dma16(srcF[i], base + C::R_BYTES + (wave + NW * i) * 1024);
-            srcF[i] += stepF[i];
+            dma16(wbase + (size_t)offF[i], base + C::R_BYTES + (wave + NW * i) * 1024);
+            offF[i] += stepF[i];
         }
     };
 
@@ -698,7 +704,11 @@ int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, hipStrea
 }
 
 bool esmm16_dma_supported(const EsmmArgs& a) {
-    return a.w_dt == a.x_dt && (a.in_dim % 32) == 0 && (a.out_dim % 8) == 0 &&
+    // the copies address their operands as base + 32-bit byte offset: the row operand and one expert's weights
+    // must each stay below 4 GiB
+    const size_t x_rows = (size_t)a.r.T * (a.x_per_slot ? a.r.k : 1);
+    const bool small = x_rows * a.in_dim * 2 < ((size_t)1 << 32) && (size_t)a.in_dim * a.out_dim * 2 < ((size_t)1 << 32);
+    return small && a.w_dt == a.x_dt && (a.in_dim % 32) == 0 && (a.out_dim % 8) == 0 &&
            (a.out_dt == a.x_dt || a.out_dt == HEXA_F32);
 }
 
@@ -732,13 +742,20 @@ int launch_estmm16_dma(const EstmmArgs& a, hipStream_t st) {
 
 // The column sums ride on the store loop of the per-slot, 16-bit-result kernels (not
 // the 128x384 tile, whose rows have 48 pieces); the pipelined kernel has its own.
+// The pipelined persistent kernel runs whatever it covers (option "pipe": 2 = never, 1 = also when a tile shape is
+// forced); the one-tile kernels run the rest.
+static bool use_pipe(const EsmmArgs& a) {
+    const int o = option(OPT_PIPE);
+    return o != 2 && (o == 1 || forced_tile() == 0) && esmm16_pipe_supported(a);
+}
+
 bool esmm16_dma_colsum_supported(const EsmmArgs& a) {
-    if (option(OPT_PIPE) == 1 && esmm16_pipe_supported(a)) return a.out_per_slot && a.r.k <= 8;
+    if (use_pipe(a)) return a.out_per_slot && a.r.k <= 8;
     return esmm16_dma_supported(a) && a.out_dt == a.x_dt && a.out_per_slot && a.r.k <= 8 && forced_tile() != 7;
 }
 
 int launch_esmm16_dma(const EsmmArgs& a, hipStream_t st) {
-    if (option(OPT_PIPE) == 1 && esmm16_pipe_supported(a)) return launch_esmm16_pipe(a, st);
+    if (use_pipe(a)) return launch_esmm16_pipe(a, st);
     if (forced_tile() == 7) return launch_esmm_dma_c<CfgW>(a, false, st);
     switch (pick_esmm_tile((long)a.r.T * a.r.k, a.out_dim, a.in_dim)) {
         case 2: return launch_esmm_dma_c<CfgL>(a, true, st);

@@ -43,7 +43,11 @@ typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
 
 constexpr int PIPE_MAX_ROUNDS = 256;   // tiles one workgroup may walk (their records are kept in LDS)
 
-using CfgP = Cfg<2, 2, 2, 2, 3, 3, 64>;   // 128 x 128: 4 multiply wavefronts of 64 x 64, 3 stages of 64 contraction indices
+#ifndef PIPE_WR
+#define PIPE_WR 2
+#define PIPE_RB 2
+#endif
+using CfgP = Cfg<PIPE_WR, 2, PIPE_RB, 2, 3, 3, 64>;   // 128 x 128: 4 multiply wavefronts of 64 x 64, 3 stages of 64 contraction indices
 
 // LDS accesses with the constant part of the address as the instruction's immediate offset (0..65535), so
 // that one address register serves a whole unrolled group of accesses
@@ -79,9 +83,10 @@ template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
 __device__ __forceinline__ void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-__device__ __forceinline__ u32x4 global_load128_async(const void* p) {
+// 16 bytes from base + off (a scalar base and a 32-bit lane offset: one address register per lane)
+__device__ __forceinline__ u32x4 global_load128_async(const void* base, unsigned off) {
     u32x4 r;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r) : "v"(p));
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(off), "s"(base));
     return r;
 }
 
@@ -93,7 +98,11 @@ struct PipeK {
     int wg_per_xcd;       // workgroups per XCD (grid = 8 * wg_per_xcd)
 };
 
-constexpr int PIPE_COPY_WAVES = 8, PIPE_STORE_WAVES = 4;
+#ifndef PIPE_CW
+#define PIPE_CW 4
+#define PIPE_SW 8
+#endif
+constexpr int PIPE_COPY_WAVES = PIPE_CW, PIPE_STORE_WAVES = PIPE_SW;
 
 template <typename C> struct PipeLds {
     static constexpr int CP = C::BN * 2 + 16;                 // pitch of a staged 16-bit result row
@@ -243,11 +252,17 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
     if (wave < NW + CW) {
         // =========================== copy wavefronts ===========================
         const int cw = wave - NW;
-        const char* srcR[R_CPW]; int stepR[R_CPW];
-        const char* srcF[F_CPW]; int stepF[F_CPW];
+        // sources as a base every lane shares plus a 32-bit byte offset per lane: the copy instruction reads one address
+        // register per lane instead of two, which matters next to wavefronts that issue MFMAs back to back; lanes with
+        // nothing to fetch re-read the first bytes of the tensor (what they produce is never stored)
+        const char* const xbase = reinterpret_cast<const char*>(p.x);
+        const char* wbase = reinterpret_cast<const char*>(p.w);
+        unsigned srcR[R_CPW]; int stepR[R_CPW];
+        unsigned srcF[F_CPW]; int stepF[F_CPW];
         auto set_sources = [&](int r) {   // this lane's copy sources for tile r (its token ids are in LDS)
             const Rec rec = tile_rec(r);
             const int e = rec.e, rows = rec.rows, s = rec.s, n0 = rec.nt * BN;
+            wbase = reinterpret_cast<const char*>(p.w) + (size_t)e * K * N * 2;
             int rowi[R_CPW], kci[R_CPW], toki[R_CPW];
 #pragma unroll
             for (int i = 0; i < R_CPW; ++i) {
@@ -260,7 +275,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
                 int tok = toki[i];
                 asm volatile("" : "+v"(tok));
                 const bool ok = rowi[i] < rows;
-                srcR[i] = ok ? reinterpret_cast<const char*>(p.x) + (((size_t)p.x_slot_rows * s + tok) * K + kci[i] * 8) * 2 : zero;
+                srcR[i] = ok ? (unsigned)((((size_t)p.x_slot_rows * s + tok) * K + kci[i] * 8) * 2) : 0u;
                 stepR[i] = ok ? BK * 2 : 0;
             }
 #pragma unroll
@@ -270,14 +285,14 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
                     ks_lane<BN>(cw + CW * i, lane, kk, ch);
                     const int n = n0 + ch * 8;
                     const bool ok = n < N;
-                    srcF[i] = ok ? reinterpret_cast<const char*>(p.w) + (((size_t)e * K + kk) * N + n) * 2 : zero;
+                    srcF[i] = ok ? (unsigned)(((size_t)kk * N + n) * 2) : 0u;
                     stepF[i] = ok ? BK * N * 2 : 0;
                 } else {         // w[e][n][k], KC
                     int row, kc;
                     kc_lane<BK>(cw + CW * i, lane, row, kc);
                     const int n = n0 + row;
                     const bool ok = n < N;
-                    srcF[i] = ok ? reinterpret_cast<const char*>(p.w) + (((size_t)e * N + n) * K + kc * 8) * 2 : zero;
+                    srcF[i] = ok ? (unsigned)(((size_t)n * K + kc * 8) * 2) : 0u;
                     stepF[i] = ok ? BK * 2 : 0;
                 }
             }
@@ -286,12 +301,12 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
             char* base = smem + stage * C::STAGE_BYTES;
 #pragma unroll
             for (int i = 0; i < R_CPW; ++i) {
-                dma16(srcR[i], base + (cw + CW * i) * 1024);
+                dma16(xbase + (size_t)srcR[i], base + (cw + CW * i) * 1024);
                 srcR[i] += stepR[i];
             }
 #pragma unroll
             for (int i = 0; i < F_CPW; ++i) {
-                dma16(srcF[i], base + C::R_BYTES + (cw + CW * i) * 1024);
+                dma16(wbase + (size_t)srcF[i], base + C::R_BYTES + (cw + CW * i) * 1024);
                 srcF[i] += stepF[i];
             }
         };
@@ -398,8 +413,9 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
         }
         const bool ok = rl < t.rows && t.col_ok;
         if (!ok) return;
-        const size_t off = (t.out_base + tok) * N + t.n;
-        unsigned short* outp = reinterpret_cast<unsigned short*>(t.to_ws ? p.ws : p.out);
+        // results, too, are addressed as a base every lane shares plus a 32-bit byte offset
+        const unsigned boff = (unsigned)(((t.out_base + tok) * N + t.n) * 2);
+        char* const outb = reinterpret_cast<char*>(t.to_ws ? p.ws : p.out);
         unsigned vw[4] = {val.x, val.y, val.z, val.w};
         if (ACT == HEXA_ACT_GELU_BWD) {
             const unsigned yw[4] = {y1v.x, y1v.y, y1v.z, y1v.w};
@@ -407,7 +423,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
             for (int u = 0; u < 4; ++u)
                 vw[u] = pack2<TC>(lo16<TC>(vw[u]) * gelu_grad_poly(lo16<TC>(yw[u])), hi16<TC>(vw[u]) * gelu_grad_poly(hi16<TC>(yw[u])));
         }
-        store16(reinterpret_cast<uint4*>(outp + off), make_uint4(vw[0], vw[1], vw[2], vw[3]), false);
+        store16(reinterpret_cast<uint4*>(outb + (size_t)boff), make_uint4(vw[0], vw[1], vw[2], vw[3]), false);
         if (COLSUM) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) { cs[2 * u] += lo16<TC>(vw[u]); cs[2 * u + 1] += hi16<TC>(vw[u]); }
@@ -416,7 +432,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
             unsigned aw[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) aw[u] = pack2<TC>(gelu_poly(lo16<TC>(vw[u])), gelu_poly(hi16<TC>(vw[u])));
-            store16(reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(p.out_act) + off),
+            store16(reinterpret_cast<uint4*>(reinterpret_cast<char*>(p.out_act) + (size_t)boff),
                     make_uint4(aw[0], aw[1], aw[2], aw[3]), false);
         }
     };
@@ -431,9 +447,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
         for (int q = 0; q < PIECES; ++q) {
             asm volatile("" : "+v"(tok[q]));
             const bool ok = rl0 + q * PROWS < t.rows && t.col_ok;
-            const void* src = ok ? (const void*)(reinterpret_cast<const unsigned short*>(p.out_act) + (t.out_base + tok[q]) * N + t.n)
-                                 : (const void*)zero;
-            y[q] = global_load128_async(src);
+            y[q] = global_load128_async(p.out_act, ok ? (unsigned)(((t.out_base + tok[q]) * N + t.n) * 2) : 0u);
         }
     };
     // column sums of the tile just stored: the lanes of a wavefront that hold the same piece, then (after the
@@ -451,6 +465,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) cs[u] = 0.f;
+        lds_wait();                                      // the sums are in LDS before this wavefront reaches the barrier
     };
     auto write_colsum = [&](const TileCtx& t) {
         if (et < BN) {
@@ -540,6 +555,10 @@ bool esmm16_pipe_supported(const EsmmArgs& a) {
     if (!(a.w_dt == a.x_dt && a.out_dt == a.x_dt && (a.in_dim % C::BKC) == 0 && a.in_dim >= (2 * C::STAGES - 2) * C::BKC && (a.out_dim % 8) == 0))
         return false;
     if (a.accumulate || a.r.k > 8) return false;
+    // copies address their operands as base + 32-bit byte offset
+    if ((size_t)a.r.T * (a.x_per_slot ? a.r.k : 1) * a.in_dim * 2 >= ((size_t)1 << 32) || (size_t)a.in_dim * a.out_dim * 2 >= ((size_t)1 << 32) ||
+        (size_t)a.r.T * a.r.k * a.out_dim * 2 >= ((size_t)1 << 32))
+        return false;
     if (!(a.out_per_slot || a.r.k == 1 || a.slot_ws != nullptr)) return false;      // every slot in one launch
     if (a.colsum && !(a.act == HEXA_ACT_GELU_BWD)) return false;
     const long total_ub = (long)a.r.k * a.r.mt_ub * div_up(a.out_dim, C::BN);

@@ -87,7 +87,8 @@ int launch_esmm32(const EsmmArgs& a, hipStream_t s);
 // can be changed at run time with hexa_set_option.
 enum Opt {
     OPT_TILE,           // HEXA_MOE_TILE: tile configuration of the 16-bit fast path (see gemm16_dma.hip)
-    OPT_PIPE,           // HEXA_MOE_PIPE: 1 = pipelined persistent ESMM kernel (multiply, copy and store wavefronts side by side)
+    OPT_PIPE,           // HEXA_MOE_PIPE: the pipelined persistent ESMM kernel (multiply, copy and store wavefronts side by side) runs
+                        // whatever it covers; 2 = never, 1 = also when a tile shape is forced
     OPT_GENERAL,        // HEXA_MOE_GENERAL_KERNELS: 1 = general 16-bit kernels instead of the fast path
     OPT_ESMM_MAP,       // HEXA_ESMM_MAP: 2 = runs of tiles per XCD instead of one contiguous eighth of the tiles per XCD
     OPT_ESMM_GROUP,     // HEXA_ESMM_GROUP: row tiles per XCD run

@@ -10,7 +10,7 @@ from oracle import hexa_oracle as O
 pytestmark = pytest.mark.gpu
 
 SETTINGS = [{"tile": t} for t in range(1, 12)] + [
-    {"pipe": 1}, {"tile": 12}, {"tile": 13},
+    {"pipe": 1}, {"pipe": 2}, {"tile": 12}, {"tile": 13},
     {"esmm_map": 2}, {"esmm_map": 2, "esmm_group": 16}, {"estmm_group": 1}, {"estmm_group": 4}, {"estmm_group": 12}, {"esmm_stream": 1}, {"general_kernels": 1},
 ]
 ALL = ("tile", "pipe", "esmm_map", "esmm_group", "estmm_group", "esmm_stream", "general_kernels")
@@ -30,10 +30,13 @@ def knobs():
 
 @pytest.mark.parametrize("cfg", SETTINGS, ids=lambda c: ",".join(f"{k}={v}" for k, v in c.items()))
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_variant(dev, knobs, cfg, dtype):
+@pytest.mark.parametrize("dims", [(2300, 192, 392), (1700, 256, 320)], ids=["192x392", "256x320"])
+def test_variant(dev, knobs, cfg, dtype, dims):
+    """The second pair of dimensions (contractions of 256 and 320: multiples of 64, at least 256) is one the pipelined
+    persistent kernel covers, in both directions; the first one it leaves to the one-tile kernels."""
     from hexa_moe import _lib, ops
     knobs(cfg)
-    T, d_in, d_out, E, k = 2300, 192, 392, 6, 2
+    (T, d_in, d_out), E, k = dims, 6, 2
     g = gen(5)
     routing = make_routing(T, E, k, seed=6, skew="zipf", empty=1)
     _, offsets, token_ids = O.route_build(routing, E)

@@ -90,6 +90,80 @@ __device__ __forceinline__ u32x4 global_load128_async(const void* base, unsigned
     return r;
 }
 
+// One stage's products for a wavefront that does nothing else: the fragments of contraction step ks+1 are read
+// from LDS while the MFMAs of step ks run (with one such wavefront per SIMD there is no neighbour to fill the
+// gap between a step's reads and its first MFMA: read-then-multiply keeps the matrix pipeline at about 60 %).
+// All reads are inline assembly and return in order: the wait before step ks allows exactly the reads of step
+// ks+1 to be outstanding, and every fragment passes through an empty statement behind that wait.
+template <int N> __device__ __forceinline__ void lds_wait_but() { asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory"); }
+template <typename TC, typename C, bool F_KS>
+__device__ __forceinline__ void mma_stage_ahead(unsigned tileR, unsigned tileF, int wr, int wf, int lane, f32x16 (&acc)[C::FB][C::RB]) {
+    using V = typename Mfma<TC>::V;
+    constexpr int RW = 32 * C::RB, FW = 32 * C::FB, KD = C::BKC, NKS = KD / 16;
+    constexpr int READS = C::RB + (F_KS ? 2 * C::FB : C::FB);      // LDS read instructions per contraction step
+    union Frag { V v; u32x4 q; s16x4 h[2]; };
+    Frag f[2][C::FB], r[2][C::RB];
+    // what does not depend on the step: the row of a KC fragment and its swizzle, the column part of a KS one
+    unsigned rbase[C::RB]; int rsw[C::RB];
+#pragma unroll
+    for (int i = 0; i < C::RB; ++i) {
+        const int row = wr * RW + i * 32 + (lane & 31);
+        rbase[i] = tileR + row * (2 * KD);
+        rsw[i] = kc_swizzle<KD>(row);
+    }
+    unsigned fbase[C::FB]; int fsw[C::FB];
+    const int grp = lane >> 4, sl = lane & 15;
+#pragma unroll
+    for (int j = 0; j < C::FB; ++j) {
+        if (F_KS) {
+            const int col = wf * FW + j * 32 + (grp & 1) * 16 + (sl & 3) * 4;
+            fbase[j] = tileF + (col & 7) * 2;
+            fsw[j] = col >> 3;
+        } else {
+            const int row = wf * FW + j * 32 + (lane & 31);
+            fbase[j] = tileF + row * (2 * KD);
+            fsw[j] = kc_swizzle<KD>(row);
+        }
+    }
+    auto read_step = [&](int ks, Frag (&fs)[C::FB], Frag (&rs)[C::RB]) {
+        const int kch = ks * 2 + (lane >> 5);
+#pragma unroll
+        for (int j = 0; j < C::FB; ++j) {
+            if (F_KS) {
+                const int k = ks * 16 + (grp >> 1) * 8 + (sl >> 2);
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int kk = k + half * 4;
+                    fs[j].h[half] = lds_read_tr16(fbase[j] + kk * (2 * C::BN) + ((fsw[j] ^ ((kk & 3) << 2)) * 16));
+                }
+            } else {
+                fs[j].q = lds_read128_async(fbase[j] + ((kch ^ fsw[j]) * 16));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C::RB; ++i) rs[i].q = lds_read128_async(rbase[i] + ((kch ^ rsw[i]) * 16));
+    };
+    read_step(0, f[0], r[0]);
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+        const int cur = ks & 1;
+        if (ks + 1 < NKS) {
+            read_step(ks + 1, f[cur ^ 1], r[cur ^ 1]);
+            lds_wait_but<READS>();
+        } else {
+            lds_wait_but<0>();
+        }
+#pragma unroll
+        for (int j = 0; j < C::FB; ++j) asm volatile("" : "+v"(f[cur][j].q));
+#pragma unroll
+        for (int i = 0; i < C::RB; ++i) asm volatile("" : "+v"(r[cur][i].q));
+#pragma unroll
+        for (int j = 0; j < C::FB; ++j)
+#pragma unroll
+            for (int i = 0; i < C::RB; ++i) acc[j][i] = Mfma<TC>::run(f[cur][j].v, r[cur][i].v, acc[j][i]);
+    }
+}
+
 template <typename TC> __device__ __forceinline__ float lo16(unsigned w) { return from_bits16<TC>(w & 0xffff); }
 template <typename TC> __device__ __forceinline__ float hi16(unsigned w) { return from_bits16<TC>(w >> 16); }
 
@@ -190,8 +264,8 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
         for (int r = 0; r < ntiles; ++r) {
             for (int kt = 0; kt < nk; ++kt) {
                 barrier_nofence();                       // the copies of this step have landed
-                const char* base = smem + stage * C::STAGE_BYTES;
-                mma_stage<TC, C, W_IN_OUT, false>(base, base + C::R_BYTES, wr, wf, lane, acc);
+                const unsigned base = lds0 + stage * C::STAGE_BYTES;
+                mma_stage_ahead<TC, C, W_IN_OUT>(base, base + C::R_BYTES, wr, wf, lane, acc);
                 stage = stage + 1 == STAGES ? 0 : stage + 1;
             }
             barrier_nofence();                           // (A) the store wavefronts are done with the staging area

@@ -183,8 +183,8 @@ template <typename C> struct PipeLds {
     static constexpr int STAGING_AT = C::STAGE_AREA;
     static constexpr int TOK_AT = STAGING_AT + C::BM * CP;    // 3 x BM token ids
     static constexpr int BIAS_SLOT = 1024;                    // one wavefront copy (64 lanes x 16 bytes) per slot
-    static constexpr int BIAS_AT = TOK_AT + 3 * C::BM * 4;    // 2 slots of raw bias elements (BN x 4 bytes used at most)
-    static constexpr int INFO_AT = BIAS_AT + 2 * BIAS_SLOT;   // PIPE_MAX_ROUNDS x int4
+    static constexpr int BIAS_AT = TOK_AT + 3 * C::BM * 4;    // 3 slots of raw bias elements (BN x 4 bytes used at most)
+    static constexpr int INFO_AT = BIAS_AT + 3 * BIAS_SLOT;   // PIPE_MAX_ROUNDS x int4
     static constexpr int RED_AT = INFO_AT + PIPE_MAX_ROUNDS * 16;   // column-sum partials: store wavefronts x BN floats
     static constexpr int SINK_AT = RED_AT + PIPE_STORE_WAVES * C::BN * 4;    // 256 bytes nobody reads (filler copies)
     static constexpr int BYTES = SINK_AT + 256;
@@ -272,7 +272,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
             // accumulators (+ bias, rounded) -> staging area
             constexpr int RW = 32 * C::RB, FW = 32 * C::FB;
             const int nl0 = wf * FW + 4 * (lane >> 5);            // + j * 32 + 8 * gq
-            const unsigned bias_at = lds0 + L::BIAS_AT + (r & 1) * L::BIAS_SLOT + nl0 * bias_esz;
+            const unsigned bias_at = lds0 + L::BIAS_AT + (r % 3) * L::BIAS_SLOT + nl0 * bias_esz;
             const unsigned stg = lds0 + L::STAGING_AT + (wr * RW + (lane & 31)) * CP + nl0 * 2;   // + i * 32 * CP
             float bv[C::FB * 4][4];
 #pragma unroll
@@ -400,7 +400,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
                 const int n = rec.nt * BN + lane * (16 / bias_esz);
                 const bool ok = lane < BN * bias_esz / 16 && n < N;
                 const void* bsrc = ok ? (const void*)(reinterpret_cast<const char*>(p.bias) + ((size_t)rec.e * N + n) * bias_esz) : (const void*)zero;
-                __builtin_amdgcn_global_load_lds((glb_ptr_t)bsrc, (lds_ptr_t)(smem + L::BIAS_AT + (r & 1) * L::BIAS_SLOT), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((glb_ptr_t)bsrc, (lds_ptr_t)(smem + L::BIAS_AT + (r % 3) * L::BIAS_SLOT), 16, 0, 0);
             } else {
                 __builtin_amdgcn_global_load_lds((glb_ptr_t)zero, (lds_ptr_t)(smem + L::SINK_AT), 4, 0, 0);
             }
@@ -432,13 +432,19 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
             for (int kt = 0; kt < nk; ++kt, ++g) {
                 // the copies of step g have landed when at most the groups of the later steps are outstanding
                 wait_groups<CPW, STAGES - 2>((int)min(total_steps - 1 - g, (long)(STAGES - 2)));
-                barrier_nofence();                       // publishes stage g; everyone is done reading stage g-1
+                // A tile's first step: the stage to refill was read in the previous tile's last step, which barrier
+                // (A) has closed, and the ring slots the next tile's token ids and bias go to were last used two tiles
+                // ago -- so these copies are issued BEFORE the step's barrier, while the multiply wavefronts are
+                // still staging the previous tile's result.
+                const bool early = kt == 0;
+                if (!early) barrier_nofence();           // publishes stage g; everyone is done reading stage g-1
                 if (kt == 0 && r + 1 < ntiles) fetch_meta(r + 1);
                 if (issued < total_steps) {
                     if (kt == nk - (STAGES - 1)) set_sources(r + 1);   // the next steps belong to the next tile
                     issue((int)(issued % STAGES));
                     ++issued;
                 }
+                if (early) barrier_nofence();
             }
             barrier_nofence();                           // (A)
         }

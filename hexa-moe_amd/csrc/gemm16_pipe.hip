@@ -31,6 +31,7 @@
 // Replaces esmm_shared_tensor_kernel_vectorized_accum_half (kernels/esmm_half.cu) and the ESMM task of the
 // fused backward kernels (kernels/fused_ops_half.cu) for the cases above.
 #include <algorithm>
+#include <type_traits>
 #include <utility>
 
 #include "dma_common.h"
@@ -167,6 +168,22 @@ __device__ __forceinline__ void mma_stage_ahead(unsigned tileR, unsigned tileF, 
 template <typename TC> __device__ __forceinline__ float lo16(unsigned w) { return from_bits16<TC>(w & 0xffff); }
 template <typename TC> __device__ __forceinline__ float hi16(unsigned w) { return from_bits16<TC>(w >> 16); }
 
+// GELU and GELU' of a value that has been rounded to bf16 are functions of 16 bits.  The store wavefronts look them up
+// in a table the workgroup builds at its start instead of evaluating them: every magnitude from 2^-14 up to (not
+// including) 8, both signs -- LUT_R entries per sign, the polynomial's own results (so nothing changes in any bit),
+// as bf16 for GELU and as fp32 for GELU' (which is multiplied before rounding).  A piece with a value outside that
+// range (zeros, |x| >= 8, NaN) takes the polynomial: one wavefront-wide branch per 16-byte piece.  The fused
+// epilogues are bound by their vector instructions (about 18 and 31 per element): a lookup is 6.
+constexpr unsigned LUT_M_LO = 0x3880, LUT_M_HI = 0x4100, LUT_R = LUT_M_HI - LUT_M_LO;
+template <typename TC, int ACT> constexpr int pipe_lut_bytes() {
+    return !std::is_same<TC, __bf16>::value ? 0 : ACT == HEXA_ACT_GELU ? 2 * LUT_R * 2 : ACT == HEXA_ACT_GELU_BWD ? 2 * LUT_R * 4 : 0;
+}
+__device__ __forceinline__ unsigned lds_read_u16_async(unsigned addr) {
+    unsigned r;
+    asm volatile("ds_read_u16 %0, %1" : "=v"(r) : "v"(addr));
+    return r;
+}
+
 struct PipeK {
     EsmmK e;
     int wg_per_xcd;       // workgroups per XCD (grid = 8 * wg_per_xcd)
@@ -178,7 +195,8 @@ struct PipeK {
 #endif
 constexpr int PIPE_COPY_WAVES = PIPE_CW, PIPE_STORE_WAVES = PIPE_SW;
 
-template <typename C> struct PipeLds {
+// LUT: bytes of the activation table behind everything else (0 = none)
+template <typename C, int LUT = 0> struct PipeLds {
     static constexpr int CP = C::BN * 2 + 16;                 // pitch of a staged 16-bit result row
     static constexpr int STAGING_AT = C::STAGE_AREA;
     static constexpr int TOK_AT = STAGING_AT + C::BM * CP;    // 3 x BM token ids
@@ -187,7 +205,9 @@ template <typename C> struct PipeLds {
     static constexpr int INFO_AT = BIAS_AT + 3 * BIAS_SLOT;   // PIPE_MAX_ROUNDS x int4
     static constexpr int RED_AT = INFO_AT + PIPE_MAX_ROUNDS * 16;   // column-sum partials: store wavefronts x BN floats
     static constexpr int SINK_AT = RED_AT + PIPE_STORE_WAVES * C::BN * 4;    // 256 bytes nobody reads (filler copies)
-    static constexpr int BYTES = SINK_AT + 256;
+    static constexpr int LUT_AT = SINK_AT + 256;
+    static constexpr int BYTES = LUT_AT + LUT;
+    static_assert(BYTES <= 160 * 1024, "LDS of a CU");
     static_assert(C::BN * 4 <= BIAS_SLOT, "bias slot");
 };
 
@@ -200,7 +220,8 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
     constexpr int R_CPW = C::R_COPIES / CW, F_CPW = C::F_COPIES / CW, CPW = R_CPW + F_CPW;   // copies per copy wavefront and stage
     static_assert(C::R_COPIES % CW == 0 && C::F_COPIES % CW == 0, "copies must divide evenly over the copy wavefronts");
     static_assert(BM <= 64 * CW, "at most one 64-id copy per copy wavefront");
-    using L = PipeLds<C>;
+    constexpr int LUT = pipe_lut_bytes<TC, ACT>();
+    using L = PipeLds<C, LUT>;
     constexpr int CP = L::CP;
     constexpr int LPR = BN / 8;                         // 16-byte pieces per staged row
     constexpr int PIECES = BM * LPR / NTS;              // pieces per store lane and tile
@@ -237,6 +258,15 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
         const int s = p.slot_begin + sl;
         const int4 rec = p.tile_info[(size_t)s * p.mt_ub + (mtg - cum[sl])];
         sInfo[i] = make_int4(rec.x, rec.y, rec.z | ((mtg - cum[sl]) << 10), (s << 24) | nt);
+    }
+    if constexpr (LUT > 0) {
+        // entry sign * LUT_R + (magnitude bits - LUT_M_LO): what the polynomial gives for exactly that bf16 value
+        for (unsigned i = tid; i < 2 * LUT_R; i += NT_ALL) {
+            const unsigned sign = i >= LUT_R ? 1u : 0u;
+            const float xv = from_bits16<TC>((unsigned short)((sign << 15) | (LUT_M_LO + i - sign * LUT_R)));
+            if (ACT == HEXA_ACT_GELU) reinterpret_cast<unsigned short*>(smem + L::LUT_AT)[i] = (unsigned short)(pack2<TC>(gelu_poly(xv), 0.f) & 0xffff);
+            else reinterpret_cast<float*>(smem + L::LUT_AT)[i] = gelu_grad_poly(xv);
+        }
     }
     __syncthreads();
 
@@ -479,6 +509,17 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
     // earlier pieces (a store is skipped when no lane of the wavefront has a valid row, so their number is not
     // fixed): allowing PIECES-1-q outstanding operations waits for that load in every case.
     const unsigned stg_lane = lds0 + L::STAGING_AT + rl0 * CP + c * 16;
+    // table positions of the eight 16-bit values of a piece; `far` = the largest distance from the table's first
+    // magnitude (unsigned: a magnitude below it wraps to a huge one), so far >= LUT_R says some value is outside
+    auto lut_index = [&](const unsigned (&w)[4], unsigned (&idx)[8], unsigned& far) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const unsigned tl = (w[u] & 0x7fffu) - LUT_M_LO, th = ((w[u] >> 16) & 0x7fffu) - LUT_M_LO;
+            far = max(far, max(tl, th));
+            idx[2 * u] = tl + ((w[u] >> 15) & 1u) * LUT_R;
+            idx[2 * u + 1] = th + (w[u] >> 31) * LUT_R;
+        }
+    };
     auto piece = [&](const TileCtx& t, auto qc, u32x4 y1v) {
         constexpr int q = decltype(qc)::value;
         const int rl = rl0 + q * PROWS;
@@ -499,9 +540,28 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
         unsigned vw[4] = {val.x, val.y, val.z, val.w};
         if (ACT == HEXA_ACT_GELU_BWD) {
             const unsigned yw[4] = {y1v.x, y1v.y, y1v.z, y1v.w};
+            bool looked_up = false;
+            if constexpr (LUT > 0) {
+                unsigned idx[8], far = 0;
+                lut_index(yw, idx, far);
+                if (__builtin_amdgcn_ballot_w64(far >= LUT_R) == 0) {   // every value of the wavefront's pieces is in the table
+                    unsigned g[8];
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
-                vw[u] = pack2<TC>(lo16<TC>(vw[u]) * gelu_grad_poly(lo16<TC>(yw[u])), hi16<TC>(vw[u]) * gelu_grad_poly(hi16<TC>(yw[u])));
+                    for (int j = 0; j < 8; ++j) g[j] = lds_read_i32(lds0 + L::LUT_AT + idx[j] * 4);
+                    lds_wait();
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) asm volatile("" : "+v"(g[j]));
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+                        vw[u] = pack2<TC>(lo16<TC>(vw[u]) * __uint_as_float(g[2 * u]), hi16<TC>(vw[u]) * __uint_as_float(g[2 * u + 1]));
+                    looked_up = true;
+                }
+            }
+            if (!looked_up) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    vw[u] = pack2<TC>(lo16<TC>(vw[u]) * gelu_grad_poly(lo16<TC>(yw[u])), hi16<TC>(vw[u]) * gelu_grad_poly(hi16<TC>(yw[u])));
+            }
         }
         store16(reinterpret_cast<uint4*>(outb + (size_t)boff), make_uint4(vw[0], vw[1], vw[2], vw[3]), false);
         if (COLSUM) {
@@ -510,8 +570,26 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
         }
         if (ACT == HEXA_ACT_GELU) {   // applied to the value as stored (rounded), like act(y1) on the tensor
             unsigned aw[4];
+            bool looked_up = false;
+            if constexpr (LUT > 0) {
+                unsigned idx[8], far = 0;
+                lut_index(vw, idx, far);
+                if (__builtin_amdgcn_ballot_w64(far >= LUT_R) == 0) {
+                    unsigned g[8];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) aw[u] = pack2<TC>(gelu_poly(lo16<TC>(vw[u])), gelu_poly(hi16<TC>(vw[u])));
+                    for (int j = 0; j < 8; ++j) g[j] = lds_read_u16_async(lds0 + L::LUT_AT + idx[j] * 2);
+                    lds_wait();
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) asm volatile("" : "+v"(g[j]));
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) aw[u] = g[2 * u] | (g[2 * u + 1] << 16);
+                    looked_up = true;
+                }
+            }
+            if (!looked_up) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) aw[u] = pack2<TC>(gelu_poly(lo16<TC>(vw[u])), gelu_poly(hi16<TC>(vw[u])));
+            }
             store16(reinterpret_cast<uint4*>(reinterpret_cast<char*>(p.out_act) + (size_t)boff),
                     make_uint4(aw[0], aw[1], aw[2], aw[3]), false);
         }
@@ -601,7 +679,7 @@ template <typename TC, bool IO, int ACT, bool COLSUM>
 int launch_pipe_t(PipeK& pk, int grid, hipStream_t st) {
     using C = CfgP;
     auto kernel = esmm16_pipe_kernel<TC, IO, ACT, COLSUM, C>;
-    constexpr int bytes = PipeLds<C>::BYTES;
+    constexpr int bytes = PipeLds<C, pipe_lut_bytes<TC, ACT>()>::BYTES;
     if (int rc = ensure_smem(kernel, bytes)) return rc;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)), bytes, st, pk);
     HEXA_CHECK_LAUNCH("esmm16_pipe");

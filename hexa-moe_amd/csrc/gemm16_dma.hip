@@ -325,6 +325,7 @@ struct EstmmK {
     int T, k, E, M, N, mtn, ntn;
     int p_slot_rows, q_slot_rows;
     int accumulate, group;
+    int off32;           // both operands below 4 GiB and 2^24 rows: rows may be addressed as base + 32-bit offset
     long total;
     const int* plan;     // non-null: units from estmm_plan_kernel (see there); scratch holds the partial results
     float* scratch;
@@ -443,28 +444,59 @@ __global__ __launch_bounds__(C::NT, C::MINW) void estmm16_dma_kernel(EstmmK p) {
         if (lane < 32)
             __builtin_amdgcn_global_load_lds((glb_ptr_t)src, (lds_ptr_t)(sIds + (step % TOK_RING) * 32), 4, 0, 0);
     };
-    // operand tiles of one step (token ids of the step are already in LDS)
+    // operand tiles of one step (token ids of the step are already in LDS).  What does not change from step to step
+    // -- which token of the step and which column piece a lane fetches -- is worked out once; a step whose 32 tokens
+    // all exist, in a tile that lies inside the result, then costs one LDS read and ONE multiply-add per copy: the
+    // row is addressed as (base of the slot's rows: scalar) + token * pitch + column offset in 32 bits (the launcher
+    // keeps tensors of 4 GiB and more, and 2^24 rows and more, off this form).  The address arithmetic of the
+    // general form (64-bit products, a block of zeros for lanes without a row) was most of this kernel's vector
+    // instructions -- three times a plain ESMM's -- and it keeps that form for the last step of a token list and for
+    // tiles on the result's edge.
+    int kkR[C::R_CPW], chR[C::R_CPW], kkF[C::F_CPW], chF[C::F_CPW];
+    unsigned colR[C::R_CPW], colF[C::F_CPW];
+#pragma unroll
+    for (int i = 0; i < C::R_CPW; ++i) {
+        ks_lane<BM>(wave + NW * i, lane, kkR[i], chR[i]);
+        colR[i] = (unsigned)(m0 + chR[i] * 8) * 2u;
+    }
+#pragma unroll
+    for (int i = 0; i < C::F_CPW; ++i) {
+        ks_lane<BN>(wave + NW * i, lane, kkF[i], chF[i]);
+        colF[i] = (unsigned)(n0 + chF[i] * 8) * 2u;
+    }
+    const bool inner_tile = p.off32 && m0 + BM <= M && n0 + BN <= N;
+    const unsigned pitchP = (unsigned)M * 2u, pitchQ = (unsigned)N * 2u;
     auto issue_data = [&](int step, Cursor c) {
         char* base = smem + (step % STAGES) * C::STAGE_BYTES;
         const unsigned ids = lds_addr(sIds + (step % TOK_RING) * 32);
         const int end = sEnd[c.s];
-        int kkR[C::R_CPW], chR[C::R_CPW], kkF[C::F_CPW], chF[C::F_CPW];
         int tokR[C::R_CPW], tokF[C::F_CPW];
 #pragma unroll
-        for (int i = 0; i < C::R_CPW; ++i) {
-            ks_lane<BM>(wave + NW * i, lane, kkR[i], chR[i]);
-            tokR[i] = lds_read_i32(ids + 4 * kkR[i]);
-        }
+        for (int i = 0; i < C::R_CPW; ++i) tokR[i] = lds_read_i32(ids + 4 * kkR[i]);
 #pragma unroll
-        for (int i = 0; i < C::F_CPW; ++i) {
-            ks_lane<BN>(wave + NW * i, lane, kkF[i], chF[i]);
-            tokF[i] = lds_read_i32(ids + 4 * kkF[i]);
-        }
+        for (int i = 0; i < C::F_CPW; ++i) tokF[i] = lds_read_i32(ids + 4 * kkF[i]);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (inner_tile && c.r + BK <= end) {
+            const char* const pb = reinterpret_cast<const char*>(p.pm) + (size_t)p.p_slot_rows * c.s * pitchP;
+            const char* const qb = reinterpret_cast<const char*>(p.qm) + (size_t)p.q_slot_rows * c.s * pitchQ;
+#pragma unroll
+            for (int i = 0; i < C::R_CPW; ++i) {
+                int tok = tokR[i];
+                asm volatile("" : "+v"(tok));   // consumed only after the wait above
+                dma16(pb + (size_t)(__umul24((unsigned)tok, pitchP) + colR[i]), base + (wave + NW * i) * 1024);
+            }
+#pragma unroll
+            for (int i = 0; i < C::F_CPW; ++i) {
+                int tok = tokF[i];
+                asm volatile("" : "+v"(tok));
+                dma16(qb + (size_t)(__umul24((unsigned)tok, pitchQ) + colF[i]), base + C::R_BYTES + (wave + NW * i) * 1024);
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < C::R_CPW; ++i) {
             int tok = tokR[i];
-            asm volatile("" : "+v"(tok));   // consumed only after the wait above
+            asm volatile("" : "+v"(tok));
             const bool ok = (c.r + kkR[i] < end) && (m0 + chR[i] * 8 < M);
             const char* sp = ok ? reinterpret_cast<const char*>(p.pm) + (((size_t)p.p_slot_rows * c.s + tok) * M + m0 + chR[i] * 8) * 2 : zero;
             dma16(sp, base + (wave + NW * i) * 1024);
@@ -590,6 +622,8 @@ int launch_estmm_dma_c(const EstmmArgs& a, hipStream_t st) {
     p.p_slot_rows = a.p_per_slot ? a.r.T : 0;
     p.q_slot_rows = a.q_per_slot ? a.r.T : 0;
     p.accumulate = a.accumulate;
+    p.off32 = (size_t)a.r.T * a.r.k < ((size_t)1 << 24) && (size_t)a.r.T * (a.p_per_slot ? a.r.k : 1) * a.m_dim * 2 < ((size_t)1 << 32) &&
+              (size_t)a.r.T * (a.q_per_slot ? a.r.k : 1) * a.n_dim * 2 < ((size_t)1 << 32) && a.m_dim * 2 < (1 << 24) && a.n_dim * 2 < (1 << 24);
     // Runs of `group` tiles per XCD (workgroup ids go round-robin over the 8 XCDs, each with its own L2).  Runs of 3
     // row tiles (with all their column tiles) cut the launch's HBM fetch at the benchmark shape from 340 to 230 MB
     // (1.28x the operands: the Q rows of an expert are then fetched by fewer L2s) at the same time, 97 against 99 us;

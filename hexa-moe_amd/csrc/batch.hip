@@ -42,6 +42,8 @@ constexpr unsigned MASK_A = TASK_ESS | TASK_ROUTER_BWD;
 constexpr unsigned MASK_B = TASK_FIXUP | TASK_ESS_FOLD;
 constexpr unsigned MASK_C = TASK_FIXUP | TASK_COLSUM_FOLD;
 constexpr unsigned MASK_D = TASK_SUM_SLOTS | TASK_DWG_REDUCE;
+constexpr unsigned MASK_E = TASK_ESS | TASK_ROUTER_BWD | TASK_FIXUP;          // the three-launch arrangement of the depth backward
+constexpr unsigned MASK_F = TASK_ESS_FOLD | TASK_FIXUP | TASK_COLSUM_FOLD;
 
 template <typename T, unsigned MASK>
 int launch_batch(const BatchK& b, hipStream_t st) {
@@ -56,6 +58,8 @@ int launch_batch_t(const BatchK& b, unsigned kinds, hipStream_t st) {
     if ((kinds & ~MASK_D) == 0) return launch_batch<T, MASK_D>(b, st);
     if ((kinds & ~MASK_A) == 0) return launch_batch<T, MASK_A>(b, st);
     if ((kinds & ~MASK_C) == 0) return launch_batch<T, MASK_C>(b, st);
+    if ((kinds & ~MASK_E) == 0) return launch_batch<T, MASK_E>(b, st);
+    if ((kinds & ~MASK_F) == 0) return launch_batch<T, MASK_F>(b, st);
     HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "batch: no kernel for the task combination 0x%x", kinds);
 }
 
@@ -66,7 +70,7 @@ unsigned kinds_of(const SmallBatch& b) {
 }
 
 bool combination_ok(unsigned k) {
-    return (k & ~MASK_A) == 0 || (k & ~MASK_B) == 0 || (k & ~MASK_C) == 0 || (k & ~MASK_D) == 0;
+    return (k & ~MASK_A) == 0 || (k & ~MASK_B) == 0 || (k & ~MASK_C) == 0 || (k & ~MASK_D) == 0 || (k & ~MASK_E) == 0 || (k & ~MASK_F) == 0;
 }
 
 }  // namespace

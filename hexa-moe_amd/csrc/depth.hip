@@ -221,14 +221,16 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
 
     // The second-stage and elementwise kernels of this call are independent of most of what surrounds them, and a
     // launch of its own costs each of them 5-7 us: where the element type has a batch kernel they are collected
-    // as tasks and run four launches (A-D) instead of nine, each placed where the stream order allows:
-    //   A  ESS(dy) partial sums, router backward              -- before anything that needs them
-    //   B  fix-up of dW2, fold of the ESS partial sums        -- behind ESTMM dW2 (the scratch is reused by dW1)
-    //   C  fix-up of dW1, fold of db1's column sums           -- behind ESTMM dW1
-    //   D  slot sum of dx (+ the gate's share), gate dwg fold -- behind the dx kernel
+    // as tasks and run three launches instead of nine, each placed where the stream order allows:
+    //   B  ESS(dy) partial sums, router backward, fix-up of dW2     -- behind ESTMM dW2 (the scratch is reused by dW1)
+    //   C  fold of the ESS partial sums, fix-up of dW1, fold of db1's column sums   -- behind ESTMM dW1 and the gate
+    //   D  slot sum of dx (+ the gate's share), gate dwg fold       -- behind the dx kernel
+    // (option "batch" = 1 keeps ESS(dy) and the router backward in a launch of their own at the start, A, and the ESS
+    // fold in B: four launches.)
     // A launcher that cannot put its task into the batch offered (other element type, general kernels) launches it
     // on the spot, which is always in order.
     const bool batching = batch_supported(d->act_dt) && option(OPT_BATCH) != 2;
+    const bool early_a = option(OPT_BATCH) == 1;
     SmallBatch A, B, C, D;
     A.dt = B.dt = C.dt = D.dt = d->act_dt;
     struct Guard { ~Guard() { defer_targets() = DeferTargets(); } } guard;
@@ -237,13 +239,13 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
 
     // step 4: db2 = ESS(dy)
     if (db2) {
-        if (batching) { tg.ess = &A; tg.ess_fold = &B; }
+        if (batching) { tg.ess = early_a ? &A : &B; tg.ess_fold = early_a ? &B : &C; }
         RUN(hexa_ess(db2, dy, route, 0, 0, T, k, d->d_out, E, d->act_dt, d->gb2_dt, w.ess, (int64_t)8 * E * d->d_out, stream));
         tg = DeferTargets();
     }
     // the gate path, part 1: d l_aux / d logits through the softmax (and the threshold)
     if (gate_path) {
-        if (batching) tg.router_bwd = &A;
+        if (batching) tg.router_bwd = early_a ? &A : &B;
         if (d->loss == 0)
             RUN(hexa_router_backward(w.dlogits, scores, stats + E, grad_l_aux, T, E, stream));
         else

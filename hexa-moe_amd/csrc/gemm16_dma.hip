@@ -325,6 +325,7 @@ struct EstmmK {
     int T, k, E, M, N, mtn, ntn;
     int p_slot_rows, q_slot_rows;
     int accumulate, group;
+    int stream_dw;       // finished results (not the partial ones of split experts) leave with the non-temporal hint
     int off32;           // both operands below 4 GiB and 2^24 rows: rows may be addressed as base + 32-bit offset
     long total;
     const int* plan;     // non-null: units from estmm_plan_kernel (see there); scratch holds the partial results
@@ -548,6 +549,8 @@ __global__ __launch_bounds__(C::NT, C::MINW) void estmm16_dma_kernel(EstmmK p) {
     // The block leaves through LDS, PRF rows at a time (pitch BN+4 floats), so that BN/4 lanes write
     // one contiguous row of dw; 16-bit results are packed on the way out.
     const bool accumulate = p.accumulate != 0;
+    typedef __attribute__((ext_vector_type(4))) float f4;
+    typedef __attribute__((ext_vector_type(2))) unsigned u2;
     float* sC = reinterpret_cast<float*>(smem);
     constexpr int CPF = BN + 4;
     constexpr int PRF = estmm_pass_rows<C>();
@@ -587,7 +590,8 @@ __global__ __launch_bounds__(C::NT, C::MINW) void estmm16_dma_kernel(EstmmK p) {
                 if (OUT32) {
                     float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(p.dw) + off);
                     if (accumulate) { const float4 old = *dst; v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w; }
-                    *dst = v;
+                    if (p.stream_dw) { const f4 w4 = {v.x, v.y, v.z, v.w}; __builtin_nontemporal_store(w4, reinterpret_cast<f4*>(dst)); }
+                    else *dst = v;
                 } else {
                     uint2* dst = reinterpret_cast<uint2*>(reinterpret_cast<unsigned short*>(p.dw) + off);
                     if (accumulate) {
@@ -595,7 +599,9 @@ __global__ __launch_bounds__(C::NT, C::MINW) void estmm16_dma_kernel(EstmmK p) {
                         v.x += from_bits16<TC>(old.x & 0xffff); v.y += from_bits16<TC>(old.x >> 16);
                         v.z += from_bits16<TC>(old.y & 0xffff); v.w += from_bits16<TC>(old.y >> 16);
                     }
-                    *dst = pack4<TC>(v.x, v.y, v.z, v.w);
+                    const uint2 pk = pack4<TC>(v.x, v.y, v.z, v.w);
+                    if (p.stream_dw) { const u2 w2 = {pk.x, pk.y}; __builtin_nontemporal_store(w2, reinterpret_cast<u2*>(dst)); }
+                    else *dst = pk;
                 }
             }
         }
@@ -622,6 +628,7 @@ int launch_estmm_dma_c(const EstmmArgs& a, hipStream_t st) {
     p.p_slot_rows = a.p_per_slot ? a.r.T : 0;
     p.q_slot_rows = a.q_per_slot ? a.r.T : 0;
     p.accumulate = a.accumulate;
+    p.stream_dw = option(OPT_ESMM_STREAM) != 2;
     p.off32 = (size_t)a.r.T * a.r.k < ((size_t)1 << 24) && (size_t)a.r.T * (a.p_per_slot ? a.r.k : 1) * a.m_dim * 2 < ((size_t)1 << 32) &&
               (size_t)a.r.T * (a.q_per_slot ? a.r.k : 1) * a.n_dim * 2 < ((size_t)1 << 32) && a.m_dim * 2 < (1 << 24) && a.n_dim * 2 < (1 << 24);
     // Runs of `group` tiles per XCD (workgroup ids go round-robin over the 8 XCDs, each with its own L2).  Runs of 3

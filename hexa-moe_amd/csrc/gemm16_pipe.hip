@@ -85,6 +85,12 @@ template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
 }
 __device__ __forceinline__ void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 // 16 bytes from base + off (a scalar base and a 32-bit lane offset: one address register per lane)
+// 16-byte store to base + off (a base every lane shares plus a 32-bit byte offset); `streaming` (uniform) adds the
+// non-temporal hint
+__device__ __forceinline__ void global_store128(void* base, unsigned off, u32x4 v, bool streaming) {
+    if (streaming) asm volatile("global_store_dwordx4 %0, %1, %2 nt" ::"v"(off), "v"(v), "s"(base) : "memory");
+    else asm volatile("global_store_dwordx4 %0, %1, %2" ::"v"(off), "v"(v), "s"(base) : "memory");
+}
 __device__ __forceinline__ u32x4 global_load128_async(const void* base, unsigned off) {
     u32x4 r;
     asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(off), "s"(base));
@@ -234,6 +240,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int K = p.K, N = p.N, nk = K / BK;
+    const bool streaming = p.stream_out != 0;           // results leave with the non-temporal hint
 
     // ---- this workgroup's walk: XCD x owns one contiguous eighth of the valid tiles (column tiles fastest);
     // the workgroups of an XCD take its tiles round-robin, so at any time they share token rows and weights
@@ -563,7 +570,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
                     vw[u] = pack2<TC>(lo16<TC>(vw[u]) * gelu_grad_poly(lo16<TC>(yw[u])), hi16<TC>(vw[u]) * gelu_grad_poly(hi16<TC>(yw[u])));
             }
         }
-        store16(reinterpret_cast<uint4*>(outb + (size_t)boff), make_uint4(vw[0], vw[1], vw[2], vw[3]), false);
+        global_store128(outb, boff, u32x4{vw[0], vw[1], vw[2], vw[3]}, streaming);
         if (COLSUM) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) { cs[2 * u] += lo16<TC>(vw[u]); cs[2 * u + 1] += hi16<TC>(vw[u]); }
@@ -590,8 +597,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
 #pragma unroll
                 for (int u = 0; u < 4; ++u) aw[u] = pack2<TC>(gelu_poly(lo16<TC>(vw[u])), gelu_poly(hi16<TC>(vw[u])));
             }
-            store16(reinterpret_cast<uint4*>(reinterpret_cast<char*>(p.out_act) + (size_t)boff),
-                    make_uint4(aw[0], aw[1], aw[2], aw[3]), false);
+            global_store128(p.out_act, boff, u32x4{aw[0], aw[1], aw[2], aw[3]}, streaming);
         }
     };
     auto load_y1 = [&](const TileCtx& t, u32x4 (&y)[PIECES]) {
@@ -736,7 +742,7 @@ int launch_esmm16_pipe(const EsmmArgs& a, hipStream_t st) {
     p.x_slot_rows = a.x_per_slot ? a.r.T : 0;
     p.out_slot_rows = a.out_per_slot ? a.r.T : 0;
     p.bias_dt = a.bias_dt; p.out_dt = a.out_dt; p.act = a.act;
-    p.stream_out = 0; p.colsum = a.colsum; p.group = 0; p.accumulate = 0;
+    p.stream_out = option(OPT_ESMM_STREAM) != 2; p.colsum = a.colsum; p.group = 0; p.accumulate = 0;
     p.ws = (!a.out_per_slot && a.r.k > 1) ? a.slot_ws : nullptr;
     p.slot_begin = 0; p.nslots = a.r.k;
     p.total = (long)p.nslots * p.mt_ub * p.ntn;

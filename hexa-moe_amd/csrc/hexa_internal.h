@@ -93,7 +93,8 @@ enum Opt {
     OPT_ESMM_MAP,       // HEXA_ESMM_MAP: 2 = runs of tiles per XCD instead of one contiguous eighth of the tiles per XCD
     OPT_ESMM_GROUP,     // HEXA_ESMM_GROUP: row tiles per XCD run
     OPT_ESTMM_GROUP,    // HEXA_ESTMM_GROUP: row tiles per XCD run
-    OPT_ESMM_STREAM,    // HEXA_ESMM_STREAM: 1 = results stored with the streaming hint
+    OPT_ESMM_STREAM,    // HEXA_ESMM_STREAM: results stored with the streaming (non-temporal) hint: 0 = by the pipelined ESMM
+                        // kernel and ESTMM's finished results, 1 = by the one-tile ESMM kernels as well, 2 = by none
     OPT_ROUTE_KERNELS,  // HEXA_ROUTE_KERNELS: 3 = always the three-launch routing pass, 1 = one launch up to 65536 tokens
     OPT_BATCH,          // HEXA_MOE_BATCH: 2 = every small kernel of the depth backward in a launch of its own, 1 = four batch launches instead of three
     OPT_FFN_FUSED,      // HEXA_MOE_FFN_FUSED: 1 = hexa_moe_depth_forward runs fc1, GELU and fc2 in one kernel where it is covered

@@ -290,10 +290,24 @@ __device__ __forceinline__ void estmm_fixup_body(const FixupK& p, int block) {
         if (c < n) { v.x += w[c].x; v.y += w[c].y; v.z += w[c].z; v.w += w[c].w; }
     }
     const size_t o = (size_t)e * p.mn + i;
-    store_out(p.dw, o, v.x, p.dw_dt, p.accumulate != 0);
-    store_out(p.dw, o + 1, v.y, p.dw_dt, p.accumulate != 0);
-    store_out(p.dw, o + 2, v.z, p.dw_dt, p.accumulate != 0);
-    store_out(p.dw, o + 3, v.w, p.dw_dt, p.accumulate != 0);
+    if (!p.accumulate) {   // one store of the four results (mn is a multiple of 4, so the piece is aligned)
+        typedef __attribute__((ext_vector_type(4))) float f4;
+        typedef __attribute__((ext_vector_type(2))) unsigned u2;
+        if (p.dw_dt == HEXA_F32) {
+            f4 w4 = {v.x, v.y, v.z, v.w};
+            *reinterpret_cast<f4*>(reinterpret_cast<float*>(p.dw) + o) = w4;
+        } else {
+            union { __bf16 b[4]; _Float16 h[4]; u2 w; } pk;   // the conversions of store_out
+            if (p.dw_dt == HEXA_BF16) { pk.b[0] = (__bf16)v.x; pk.b[1] = (__bf16)v.y; pk.b[2] = (__bf16)v.z; pk.b[3] = (__bf16)v.w; }
+            else { pk.h[0] = (_Float16)v.x; pk.h[1] = (_Float16)v.y; pk.h[2] = (_Float16)v.z; pk.h[3] = (_Float16)v.w; }
+            *reinterpret_cast<u2*>(reinterpret_cast<unsigned short*>(p.dw) + o) = pk.w;
+        }
+        return;
+    }
+    store_out(p.dw, o, v.x, p.dw_dt, true);
+    store_out(p.dw, o + 1, v.y, p.dw_dt, true);
+    store_out(p.dw, o + 2, v.z, p.dw_dt, true);
+    store_out(p.dw, o + 3, v.w, p.dw_dt, true);
 }
 
 // db[e][n] (+)= the column sums an ESMM launch left per (slot, row tile, column tile), added in tile order.

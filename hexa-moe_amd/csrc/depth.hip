@@ -154,9 +154,10 @@ extern "C" int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* 
         const bool one_launch = front3 && option(OPT_GATE_ROUTER) != 2 && T > 0 && gate_router_supported(d->d_in, E, d->act_dt);
         if (!one_launch) RUN(hexa_gate_logits(logits, x, wg, T, d->d_in, E, d->act_dt, stream));
         if (front3) {
-            // three launches for gate, router, loss, routing pass and plan: the gate's logits go straight into the
-            // router's tile (two launches above GATE_ROUTER_MAX_E experts), the router counts its own tokens for the
-            // routing pass, whose scan launch carries the loss and whose scatter launch carries the plan
+            // two launches for gate, router, loss, routing pass and plan: the gate's logits go straight into the
+            // router's tile (a launch of its own above GATE_ROUTER_MAX_E experts), the router counts its own tokens for
+            // the routing pass, whose one launch also carries the loss and the plan (above 256 experts, or with option
+            // "route_kernels" = 3: a scan launch with the loss and a scatter launch with the plan)
             RUN(router_forward_check(T, E, k, true));
             if (one_launch)
                 RUN(launch_gate_router(logits, scores, idx, x, wg, noise, d->noise_scale, T, d->d_in, E, k, d->act_dt, w.router,

@@ -95,7 +95,8 @@ enum Opt {
     OPT_ESTMM_GROUP,    // HEXA_ESTMM_GROUP: row tiles per XCD run
     OPT_ESMM_STREAM,    // HEXA_ESMM_STREAM: results stored with the streaming (non-temporal) hint: 0 = by the pipelined ESMM
                         // kernel and ESTMM's finished results, 1 = by the one-tile ESMM kernels as well, 2 = by none
-    OPT_ROUTE_KERNELS,  // HEXA_ROUTE_KERNELS: 3 = always the three-launch routing pass, 1 = one launch up to 65536 tokens
+    OPT_ROUTE_KERNELS,  // HEXA_ROUTE_KERNELS: 3 = always the three-launch routing pass (behind the router's histogram: a scan and
+                        // a scatter launch instead of one), 1 = one launch up to 65536 tokens
     OPT_BATCH,          // HEXA_MOE_BATCH: 2 = every small kernel of the depth backward in a launch of its own, 1 = four batch launches instead of three
     OPT_FFN_FUSED,      // HEXA_MOE_FFN_FUSED: 1 = hexa_moe_depth_forward runs fc1, GELU and fc2 in one kernel where it is covered
     OPT_GATE_ROUTER,    // HEXA_MOE_GATE_ROUTER: 2 = hexa_moe_depth_forward runs the gate projection and the router as two launches

@@ -97,9 +97,8 @@ __device__ void emit_tiles(const int32_t* tot, const int32_t* off, int32_t* tbas
     __syncthreads();
 }
 
-__device__ void finish_slot(const int32_t* tot, int32_t* off, int32_t* tbase, int* tmp, int E, int pad,
-                            int32_t* counts, int32_t* offsets, int4* tile_info, int32_t* tile_count,
-                            int mt_ub, int4* tile_info_l, int32_t* tile_count_l, int mt_ub_l) {
+// off[0..E] (LDS) = exclusive prefix of the totals tot[E] (LDS), each rounded up to `pad`.  tmp: 16 ints of LDS.
+__device__ void scan_offsets(const int32_t* tot, int32_t* off, int* tmp, int E, int pad) {
     const int tid = threadIdx.x;
     const int nthr = blockDim.x;
     const int chunk = (E + nthr - 1) / nthr;
@@ -114,6 +113,14 @@ __device__ void finish_slot(const int32_t* tot, int32_t* off, int32_t* tbase, in
     }
     if (tid == 0) off[E] = total_rows;
     __syncthreads();
+}
+
+__device__ void finish_slot(const int32_t* tot, int32_t* off, int32_t* tbase, int* tmp, int E, int pad,
+                            int32_t* counts, int32_t* offsets, int4* tile_info, int32_t* tile_count,
+                            int mt_ub, int4* tile_info_l, int32_t* tile_count_l, int mt_ub_l) {
+    const int tid = threadIdx.x;
+    const int nthr = blockDim.x;
+    scan_offsets(tot, off, tmp, E, pad);
     for (int e = tid; e <= E; e += nthr) {
         if (offsets) offsets[e] = off[e];
         if (counts && e < E) counts[e] = tot[e];
@@ -248,6 +255,13 @@ __global__ __launch_bounds__(256) void route_scan_loss_kernel(int32_t* __restric
 }
 
 template <typename IdxT>
+__device__ __forceinline__ void route_scatter_loop(int32_t* cursor, bool worker, int unit, int s, int unit_tokens,
+                                                   const IdxT* __restrict__ routing, int64_t token_stride,
+                                                   int64_t slot_stride, int T, int E, int nbits,
+                                                   int32_t* __restrict__ token_ids, int32_t* __restrict__ expert_ids,
+                                                   int64_t list_stride);
+
+template <typename IdxT>
 __device__ __forceinline__ void route_scatter_body(int32_t* cursor, int unit, int s, int unit_tokens,
                                                    const IdxT* __restrict__ routing, int64_t token_stride,
                                                    int64_t slot_stride, int T, int E, int units, int nbits,
@@ -260,6 +274,20 @@ __device__ __forceinline__ void route_scatter_body(int32_t* cursor, int unit, in
     const int32_t* off = offsets + (size_t)s * offsets_slot_stride;
     for (int i = lane; i < E; i += kWave) cursor[i] = off[i] + H[i];
     __syncthreads();
+    route_scatter_loop<IdxT>(cursor, true, unit, s, unit_tokens, routing, token_stride, slot_stride, T, E, nbits, token_ids,
+                             expert_ids, list_stride);
+}
+
+// The stable scatter of one unit's tokens given cursor[e] (LDS) = the list position of the unit's first token of
+// expert e.  Every wavefront of the workgroup must call it (it contains barriers); the one with `worker` set (the
+// first) does the work.
+template <typename IdxT>
+__device__ __forceinline__ void route_scatter_loop(int32_t* cursor, bool worker, int unit, int s, int unit_tokens,
+                                                   const IdxT* __restrict__ routing, int64_t token_stride,
+                                                   int64_t slot_stride, int T, int E, int nbits,
+                                                   int32_t* __restrict__ token_ids, int32_t* __restrict__ expert_ids,
+                                                   int64_t list_stride) {
+    const int lane = threadIdx.x & 63;
     const int t0 = unit * unit_tokens;
     const int t1 = min(T, t0 + unit_tokens);
     const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
@@ -268,7 +296,7 @@ __device__ __forceinline__ void route_scatter_body(int32_t* cursor, int unit, in
     for (int base = t0; base < t1; base += kWave) {   // trip count is uniform over the wavefront
         const int t = base + lane;
         long e = -1;
-        if (t < t1) e = (long)routing[(int64_t)t * token_stride + (int64_t)s * slot_stride];
+        if (worker && t < t1) e = (long)routing[(int64_t)t * token_stride + (int64_t)s * slot_stride];
         const bool valid = (e >= 0 && e < E);
         // lanes holding the same expert id: AND over the id's bits of "lanes that agree on the bit"
         unsigned long long peers = __ballot(valid);
@@ -320,6 +348,105 @@ __global__ __launch_bounds__(kWave) void route_scatter_plan_kernel(const int32_t
                                     offsets, E + 1, token_ids, expert_ids, T);
     } else if (blockIdx.y == 0 && plan) {
         estmm_plan_body(cursor, plan, offsets, E, k, plan_cap, plan_slots);
+    }
+}
+
+// Per expert, the raw per-unit counts H[u][e] summed over all units (tot) and over the units before u_split (pre,
+// may be null): 256 / E threads share an expert (E <= 256), thread group j takes the units j, j + G, ..., sixteen
+// loads in flight at a time; the partial sums meet in LDS.  part: 512 ints, tot / pre: E ints each, all LDS.
+// 256 threads.
+__device__ __forceinline__ void unit_sums(const int32_t* __restrict__ H, int E, int units, int u_split, int32_t* part,
+                                          int32_t* tot, int32_t* pre) {
+    const int tid = threadIdx.x;
+    const int G = 256 / E;
+    const int e = tid % E, j = tid / E;
+    int t = 0, q = 0;
+    if (j < G) {
+        for (int u0 = j; u0 < units; u0 += 16 * G) {
+            int v[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v[i] = u0 + i * G < units ? H[(size_t)(u0 + i * G) * E + e] : 0;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { t += v[i]; q += u0 + i * G < u_split ? v[i] : 0; }
+        }
+    }
+    part[tid] = t;
+    part[256 + tid] = q;
+    __syncthreads();
+    if (tid < E) {
+        int a = 0, b = 0;
+        for (int g = 0; g < G; ++g) { a += part[g * E + tid]; b += part[256 + g * E + tid]; }
+        tot[tid] = a;
+        if (pre) pre[tid] = b;
+    }
+    __syncthreads();
+}
+
+// Everything behind the router's per-unit histogram (raw counts, hist [k][units][E], E <= 256) in ONE launch of
+// 256-thread workgroups:
+//   [0, units * k)   scatter of one unit of one slot: the workgroup adds up the counts of the units before its own and
+//                    of all units itself (the histogram is a few tens of KB in L2), scans the experts and scatters
+//   the next k       one per slot: totals, offsets, counts, row-tile records
+//   then             the GShard loss from the router's partial sums (when l_aux is given)
+//   then             the ESTMM work plan (when plan is given), from the totals of all slots
+// No workgroup reads what another one of the launch writes, and the histogram is left as it was.
+__global__ __launch_bounds__(256) void route_finish_kernel(const int32_t* __restrict__ routing, int k, int T, int E, int units,
+                                                           int unit_tokens, int nbits, const int32_t* __restrict__ unit_hist,
+                                                           int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
+                                                           int4* __restrict__ tile_info, int32_t* __restrict__ tile_count,
+                                                           int mt_ub, int4* __restrict__ tile_info_l,
+                                                           int32_t* __restrict__ tile_count_l, int mt_ub_l,
+                                                           int32_t* __restrict__ token_ids, int32_t* __restrict__ expert_ids,
+                                                           float* __restrict__ l_aux, float* __restrict__ me,
+                                                           float* __restrict__ ce, const float* __restrict__ part_me,
+                                                           const float* __restrict__ part_cnt,
+                                                           int32_t* __restrict__ plan, int plan_cap, int plan_slots) {
+    extern __shared__ int32_t sh[];
+    __shared__ int32_t part[512];
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const int n_scatter = units * k;
+    if (b < n_scatter) {
+        const int unit = b % units, s = b / units;
+        int32_t* tot = sh;                // E
+        int32_t* pre = tot + E;           // E
+        int32_t* off = pre + E;           // E + 1
+        int32_t* cursor = off + (E + 1);  // E
+        int* tmp = cursor + E;            // 16
+        unit_sums(unit_hist + (size_t)s * units * E, E, units, unit, part, tot, pre);
+        scan_offsets(tot, off, tmp, E, 1);
+        for (int e = tid; e < E; e += 256) cursor[e] = off[e] + pre[e];
+        __syncthreads();
+        route_scatter_loop<int32_t>(cursor, tid < kWave, unit, s, unit_tokens, routing, k, 1, T, E, nbits, token_ids,
+                                    expert_ids, T);
+        return;
+    }
+    if (b < n_scatter + k) {
+        const int s = b - n_scatter;
+        int32_t* tot = sh;                // the layout of route_scan_body
+        int32_t* off = tot + E;
+        int32_t* tbase = off + (E + 1);
+        int* tmp = tbase + (E + 1);
+        unit_sums(unit_hist + (size_t)s * units * E, E, units, units, part, tot, nullptr);
+        finish_slot(tot, off, tbase, tmp, E, 1, counts + (size_t)s * E, offsets + (size_t)s * (E + 1),
+                    tile_info + (size_t)s * mt_ub, tile_count + s, mt_ub, tile_info_l + (size_t)s * mt_ub_l, tile_count_l + s,
+                    mt_ub_l);
+        return;
+    }
+    if (l_aux && b == n_scatter + k) {
+        router_loss_body(reinterpret_cast<float*>(sh), l_aux, me, ce, part_me, part_cnt, units, T, E);
+        return;
+    }
+    if (plan) {
+        int32_t* load = sh;               // 2 * E for the plan, then E of totals
+        int32_t* tot = sh + 2 * E;
+        for (int e = tid; e < E; e += 256) load[e] = 0;
+        __syncthreads();
+        for (int s = 0; s < k; ++s) {
+            unit_sums(unit_hist + (size_t)s * units * E, E, units, units, part, tot, nullptr);
+            if (tid < E) load[tid] += tot[tid];
+            __syncthreads();
+        }
+        estmm_plan_from_loads(load, plan, E, plan_cap, plan_slots);
     }
 }
 
@@ -547,6 +674,17 @@ int launch_route_from_hist(const int32_t* idx, int T, int k, int E, int32_t* rou
     hexa_route_layout_get(T, k, E, &L);
     const int units = div_up(T, unit_tokens);
     const size_t loss_lds = l_aux ? sizeof(float) * (2 * (size_t)router_loss_chunks(E) * E + 256) : 0;
+    if (E <= 256 && option(OPT_ROUTE_KERNELS) != 3) {   // one launch; the histogram stays as counted
+        const size_t lds = std::max({sizeof(int32_t) * (size_t)(4 * E + 1 + 16), scan_lds_bytes(E), loss_lds});
+        const int grid = units * k + k + (l_aux ? 1 : 0) + (plan ? 1 : 0);
+        hipLaunchKernelGGL(route_finish_kernel, dim3(grid), dim3(256), lds, st, idx, k, T, E, units, unit_tokens, ceil_log2(E),
+                           hist, route + L.counts, route + L.offsets, reinterpret_cast<int4*>(route + L.tile_info),
+                           route + L.tile_count, L.mt_ub, reinterpret_cast<int4*>(route + L.tile_info_l), route + L.tile_count_l,
+                           L.mt_ub_l, route + L.token_ids, route + L.expert_ids, l_aux, me, ce, router_ws,
+                           router_ws ? router_ws + (size_t)units * E : nullptr, plan, estmm_plan_cap(T, k, E), plan_slots);
+        HEXA_CHECK_LAUNCH("route_finish");
+        return HEXA_OK;
+    }
     hipLaunchKernelGGL(route_scan_loss_kernel, dim3(k + (l_aux ? 1 : 0)), dim3(256), std::max(scan_lds_bytes(E), loss_lds), st,
                        hist, E, units, k, route + L.counts, route + L.offsets, reinterpret_cast<int4*>(route + L.tile_info),
                        route + L.tile_count, L.mt_ub, reinterpret_cast<int4*>(route + L.tile_info_l), route + L.tile_count_l,

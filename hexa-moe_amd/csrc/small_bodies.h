@@ -76,10 +76,11 @@ __host__ __device__ inline int estmm_plan_cap(long T, int k, int E) {   // parts
     return (int)(c > 256 ? c : 256);
 }
 
+__device__ inline void estmm_plan_from_loads(int* sp, int* __restrict__ plan, int E, int cap, int max_slots);
+
 __device__ inline void estmm_plan_body(int* sp, int* __restrict__ plan, const int32_t* __restrict__ offsets, int E, int k,
                                        int cap, int max_slots) {
     int* load = sp;
-    int* expert_of = sp + E;          // the expert at each rank
     const int nthr = blockDim.x;
     for (int e = threadIdx.x; e < E; e += nthr) {
         int t = 0;
@@ -87,6 +88,14 @@ __device__ inline void estmm_plan_body(int* sp, int* __restrict__ plan, const in
         load[e] = t;
     }
     __syncthreads();
+    estmm_plan_from_loads(sp, plan, E, cap, max_slots);
+}
+
+// The plan from sp[0..E) = tokens per expert over all slots (written and published by the caller).
+__device__ inline void estmm_plan_from_loads(int* sp, int* __restrict__ plan, int E, int cap, int max_slots) {
+    int* load = sp;
+    int* expert_of = sp + E;          // the expert at each rank
+    const int nthr = blockDim.x;
     for (int e = threadIdx.x; e < E; e += nthr) {
         const int mine = load[e];
         int r = 0;

@@ -298,8 +298,8 @@ int hexa_moe_depth_ws_bytes(const hexa_moe_depth_desc* d, int64_t* forward_bytes
  * plan (may be NULL): 4*num_experts+1 ints that receive the work plan of the backward's ESTMM calls (as
  * hexa_estmm_plan; it depends on the routing only); hand the same buffer to hexa_moe_depth_backward and that call
  * skips making it.  (With the GShard loss and up to 240 experts the router, the loss, the routing pass and the plan
- * take three launches in all: the router counts its own tokens for the routing pass, whose scan launch finishes the
- * loss and whose scatter launch makes the plan.)
+ * take two launches in all: the router counts its own tokens for the routing pass, whose one launch scatters the
+ * tokens, finishes the loss and makes the plan.)
  * events (may be NULL): 2*n caller-owned hipEvent_t handles; pair i is recorded on `stream` around major kernel i
  * (0: fc1 + GELU, 1: fc2 and its slot sum), for callers that time kernels inside a step; NULL handles in the
  * array are skipped. */

@@ -312,6 +312,20 @@ def test_one_kernel_ffn_forward(dev, dtype, T, d, E, k, bias):
         assert_close(u, v, TOL[dtype] / 4, "parameter gradient")
 
 
+def _route_fields(blob, T, k, E):
+    """The fields of a route blob that the routing pass defines (tile records up to each slot's count)."""
+    from hexa_moe import _lib
+    L = _lib.route_layout(T, k, E)
+    b = blob.cpu()
+    out = [b[L.counts:L.counts + k * E], b[L.offsets:L.offsets + k * (E + 1)], b[L.token_ids:L.token_ids + k * T],
+           b[L.expert_ids:L.expert_ids + k * T], b[L.tile_count:L.tile_count + k], b[L.tile_count_l:L.tile_count_l + k]]
+    for s in range(k):
+        n, nl = int(b[L.tile_count + s]), int(b[L.tile_count_l + s])
+        out.append(b[L.tile_info + 4 * s * L.mt_ub:L.tile_info + 4 * (s * L.mt_ub + min(n, L.mt_ub))])
+        out.append(b[L.tile_info_l + 4 * s * L.mt_ub_l:L.tile_info_l + 4 * (s * L.mt_ub_l + min(nl, L.mt_ub_l))])
+    return [t.clone() for t in out]
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,d,E,k,train", [(2500, 256, 16, 2, True), (2300, 384, 32, 2, False), (1900, 128, 5, 3, True),
                                            (130, 264, 33, 2, True), (63, 8, 64, 1, False), (4097, 96, 7, 4, True)])
@@ -320,7 +334,8 @@ def test_gate_and_router_in_one_launch(dev, dtype, T, d, E, k, train):
     experts) against the same call with the two as separate launches (library option "gate_router" = 2): the one
     kernel repeats the gate's sums in the same order, so routing, y, l_aux and every gradient are identical -- with
     gate noise (train mode, same seed), expert counts that are no multiple of 4 or span two 32-expert blocks, and a
-    last workgroup with fewer than 64 tokens."""
+    last workgroup with fewer than 64 tokens.  Likewise the routing pass behind the router's histogram as one launch
+    (default) against a scan and a scatter launch (option "route_kernels" = 3): every field of the route is identical."""
     from hexa_moe import _lib
     lib = _lib.load()
     m = _module([d], [0], E=E, k=k, act=F.gelu, noise=1.0).to(dev).to(dtype)
@@ -332,20 +347,28 @@ def test_gate_and_router_in_one_launch(dev, dtype, T, d, E, k, train):
     dy = torch.randn(T, d, generator=g).to(dtype).to(dev)
     res = []
     try:
-        for separate in (0, 2):
-            _lib.check(lib.hexa_set_option(b"gate_router", separate), "hexa_set_option")
+        for name, value in ((b"gate_router", 0), (b"gate_router", 2), (b"route_kernels", 3)):
+            _lib.check(lib.hexa_set_option(b"gate_router", 0), "hexa_set_option")
+            _lib.check(lib.hexa_set_option(b"route_kernels", 0), "hexa_set_option")
+            _lib.check(lib.hexa_set_option(name, value), "hexa_set_option")
             torch.manual_seed(5)                      # the gate noise of both runs
             m.zero_grad(set_to_none=True)
             xi = x.clone().requires_grad_(True)
             y, l_aux = m(0, xi)
             torch.autograd.backward([y, l_aux], [dy, torch.full((), 2.0, device=dev)])
             torch.cuda.synchronize()
+            blob = next(iter(m.dispatch_params.route_pool._slots.values()))[0]
             res.append((m.dispatch_params.routing_.clone(), y.detach().clone(), l_aux.detach().clone(), xi.grad.clone(),
-                        [p.grad.clone() for p in m.parameters() if p.grad is not None]))
+                        [p.grad.clone() for p in m.parameters() if p.grad is not None], _route_fields(blob, T, k, E)))
     finally:
         _lib.check(lib.hexa_set_option(b"gate_router", 0), "hexa_set_option")
-    (ra, ya, la, dxa, ga), (rb, yb, lb, dxb, gb) = res
-    assert torch.equal(ra, rb) and torch.equal(ya, yb) and torch.equal(la, lb) and torch.equal(dxa, dxb)
-    assert len(ga) == len(gb) and len(ga) >= 3
-    for u, v in zip(ga, gb):
-        assert torch.equal(u, v)
+        _lib.check(lib.hexa_set_option(b"route_kernels", 0), "hexa_set_option")
+    ra, ya, la, dxa, ga, fa = res[0]
+    assert len(ga) >= 3
+    for rb, yb, lb, dxb, gb, fb in res[1:]:
+        assert torch.equal(ra, rb) and torch.equal(ya, yb) and torch.equal(la, lb) and torch.equal(dxa, dxb)
+        assert len(ga) == len(gb) and len(fa) == len(fb)
+        for u, v in zip(ga, gb):
+            assert torch.equal(u, v)
+        for u, v in zip(fa, fb):
+            assert torch.equal(u, v)

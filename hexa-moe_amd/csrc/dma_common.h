@@ -172,7 +172,7 @@ template <int KD = 32> __device__ __forceinline__ void kc_lane(int c, int lane, 
 }
 // KS operand of width W: copy c covers 512/W k rows; returns the k row and the column piece.
 template <int W> __device__ __forceinline__ void ks_lane(int c, int lane, int& kk, int& ch) {
-    constexpr int PPR = W / 8;               // 16-byte pieces per k row (any multiple of 4)
+    constexpr int PPR = W / 8;               // 16-byte pieces per k row (a multiple of 16: the swizzle flips bits 2 and 3)
     const int piece = 64 * c + lane;
     kk = piece / PPR;
     ch = (piece - kk * PPR) ^ ((kk & 3) << 2);

@@ -328,13 +328,15 @@ def _route_fields(blob, T, k, E):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,d,E,k,train", [(2500, 256, 16, 2, True), (2300, 384, 32, 2, False), (1900, 128, 5, 3, True),
-                                           (130, 264, 33, 2, True), (63, 8, 64, 1, False), (4097, 96, 7, 4, True)])
+                                           (130, 264, 33, 2, True), (63, 8, 64, 1, False), (4097, 96, 7, 4, True),
+                                           (700, 64, 100, 2, True), (900, 128, 240, 3, False), (500, 64, 130, 2, True)])
 def test_gate_and_router_in_one_launch(dev, dtype, T, d, E, k, train):
     """The depth call's front end with the gate projection and the router in one kernel (the default up to 64
     experts) against the same call with the two as separate launches (library option "gate_router" = 2): the one
     kernel repeats the gate's sums in the same order, so routing, y, l_aux and every gradient are identical -- with
     gate noise (train mode, same seed), expert counts that are no multiple of 4 or span two 32-expert blocks, and a
-    last workgroup with fewer than 64 tokens.  Likewise the routing pass behind the router's histogram as one launch
+    last workgroup with fewer than 64 tokens (above 64 experts the gate is a launch of its own either way).  Likewise
+    the routing pass behind the router's histogram as one launch
     (default) against a scan and a scatter launch (option "route_kernels" = 3): every field of the route is identical."""
     from hexa_moe import _lib
     lib = _lib.load()

@@ -7,6 +7,8 @@
 //   3. route_scatter one wavefront per unit again: stable rank of every token inside its
 //                    (unit, expert) group from log2(E) ballots, so a segment lists its tokens in
 //                    ascending order -- the result is a stable counting sort and is bit-reproducible.
+// Up to 256 experts launches 2 and 3 run as one (route_finish_kernel): every scatter workgroup adds up the counts of
+// the units before its own and of all units itself instead of waiting for a scan.
 // Replaces launch_count / launch_assign of the reference (kernels/shared_cuda_core.cu:126-182,
 // 284-333), which run single-workgroup launches with shared-memory atomics, two blocking copies and
 // a host-side prefix per call.
@@ -421,7 +423,9 @@ __device__ __forceinline__ void unit_sums(const int32_t* __restrict__ H, int E, 
 //   then             the GShard loss from the router's partial sums (when l_aux is given)
 //   then             the ESTMM work plan (when plan is given), from the totals of all slots
 // No workgroup reads what another one of the launch writes, and the histogram is left as it was.
-__global__ __launch_bounds__(256) void route_finish_kernel(const int32_t* __restrict__ routing, int k, int T, int E, int units,
+template <typename IdxT>
+__global__ __launch_bounds__(256) void route_finish_kernel(const IdxT* __restrict__ routing, int64_t token_stride,
+                                                           int64_t slot_stride, int k, int T, int E, int units,
                                                            int unit_tokens, int nbits, const int32_t* __restrict__ unit_hist,
                                                            int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
                                                            int4* __restrict__ tile_info, int32_t* __restrict__ tile_count,
@@ -447,8 +451,8 @@ __global__ __launch_bounds__(256) void route_finish_kernel(const int32_t* __rest
         scan_offsets(tot, off, tmp, E, 1);
         for (int e = tid; e < E; e += 256) cursor[e] = off[e] + pre[e];
         __syncthreads();
-        route_scatter_loop<int32_t>(cursor, tid < kWave, unit, s, unit_tokens, routing, k, 1, T, E, nbits, token_ids,
-                                    expert_ids, T);
+        route_scatter_loop<IdxT>(cursor, tid < kWave, unit, s, unit_tokens, routing, token_stride, slot_stride, T, E, nbits,
+                                 token_ids, expert_ids, T);
         return;
     }
     if (b < n_scatter + k) {
@@ -708,7 +712,8 @@ int launch_route_from_hist(const int32_t* idx, int T, int k, int E, int32_t* rou
     if (E <= 256 && (reinterpret_cast<uintptr_t>(hist) & 15) == 0 && option(OPT_ROUTE_KERNELS) != 3) {   // one launch; the histogram stays as counted
         const size_t lds = std::max({sizeof(int32_t) * (size_t)(4 * E + 1 + 16), scan_lds_bytes(E), loss_lds});
         const int grid = units * k + k + (l_aux ? 1 : 0) + (plan ? 1 : 0);
-        hipLaunchKernelGGL(route_finish_kernel, dim3(grid), dim3(256), lds, st, idx, k, T, E, units, unit_tokens, ceil_log2(E),
+        hipLaunchKernelGGL(route_finish_kernel<int32_t>, dim3(grid), dim3(256), lds, st, idx, (int64_t)k, (int64_t)1, k, T, E, units,
+                           unit_tokens, ceil_log2(E),
                            hist, route + L.counts, route + L.offsets, reinterpret_cast<int4*>(route + L.tile_info),
                            route + L.tile_count, L.mt_ub, reinterpret_cast<int4*>(route + L.tile_info_l), route + L.tile_count_l,
                            L.mt_ub_l, route + L.token_ids, route + L.expert_ids, l_aux, me, ce, router_ws,
@@ -771,6 +776,27 @@ extern "C" int hexa_route_build(const void* routing, int routing_is_i64, int64_t
         hipLaunchKernelGGL(route_hist_kernel<int32_t>, grid, dim3(kWave), sizeof(int32_t) * E, st,
                            (const int32_t*)routing, token_stride, slot_stride, T, E, L.units, H);
     HEXA_CHECK_LAUNCH("route_hist");
+    if (E <= 256 && option(OPT_ROUTE_KERNELS) != 3) {
+        // scan and scatter in one launch: every scatter workgroup derives its cursors from the raw histogram
+        const size_t lds = std::max(sizeof(int32_t) * (size_t)(4 * E + 1 + 16), scan_lds_bytes(E));
+        const int nwg = L.units * k + k;
+        int4* ti = reinterpret_cast<int4*>(route + L.tile_info);
+        int4* til = reinterpret_cast<int4*>(route + L.tile_info_l);
+        if (routing_is_i64)
+            hipLaunchKernelGGL(route_finish_kernel<int64_t>, dim3(nwg), dim3(256), lds, st, (const int64_t*)routing, token_stride,
+                               slot_stride, k, T, E, L.units, kUnit, nbits, H, route + L.counts, route + L.offsets, ti,
+                               route + L.tile_count, L.mt_ub, til, route + L.tile_count_l, L.mt_ub_l, route + L.token_ids,
+                               route + L.expert_ids, (float*)nullptr, (float*)nullptr, (float*)nullptr, (const float*)nullptr,
+                               (const float*)nullptr, (int32_t*)nullptr, 0, 0);
+        else
+            hipLaunchKernelGGL(route_finish_kernel<int32_t>, dim3(nwg), dim3(256), lds, st, (const int32_t*)routing, token_stride,
+                               slot_stride, k, T, E, L.units, kUnit, nbits, H, route + L.counts, route + L.offsets, ti,
+                               route + L.tile_count, L.mt_ub, til, route + L.tile_count_l, L.mt_ub_l, route + L.token_ids,
+                               route + L.expert_ids, (float*)nullptr, (float*)nullptr, (float*)nullptr, (const float*)nullptr,
+                               (const float*)nullptr, (int32_t*)nullptr, 0, 0);
+        HEXA_CHECK_LAUNCH("route_finish");
+        return HEXA_OK;
+    }
     hipLaunchKernelGGL(route_scan_kernel, dim3(k), dim3(256), scan_lds_bytes(E), st, H, E, L.units, 1,
                        route + L.counts, route + L.offsets, reinterpret_cast<int4*>(route + L.tile_info),
                        route + L.tile_count, L.mt_ub, reinterpret_cast<int4*>(route + L.tile_info_l),

@@ -26,10 +26,12 @@ CASES = [
 ]
 
 
-@pytest.fixture(params=[1, 3], ids=["one_launch", "three_launches"])
+@pytest.fixture(params=[0, 1, 3], ids=["auto", "one_launch", "three_launches"])
 def route_kernels(request):
-    """The pass runs as one launch for small token counts, else as three; both are forced in turn on every
-    case (one launch covers up to 65536 tokens and 256 experts; beyond that it is three in both runs)."""
+    """The pass runs as one launch for small token counts, else as a histogram launch and one that scans and
+    scatters (up to 256 experts), else as three; every case runs under the automatic choice, with one launch forced
+    (it covers up to 65536 tokens and 256 experts; beyond that the two- or three-launch form runs) and with three
+    forced."""
     from hexa_moe import _lib
     lib = _lib.load()
     _lib.check(lib.hexa_set_option(b"route_kernels", request.param), "hexa_set_option")

@@ -52,7 +52,7 @@ def test_abi_argument_errors_without_a_gpu():
 
 
 def test_state_dict_names_and_shapes():
-    m = _readme_module()
+    m = _readme_module(seeds=(11, 12, 13))
     sd = m.state_dict()
     want = {"batched_fc1_w.0": (8, 512, 128), "batched_fc2_w.1": (8, 512, 128), "batched_fc1_bias.0": (8, 512),
             "batched_fc2_bias.1": (8, 128), "mlp_fc1_w.0": (512, 128), "mlp_fc2_w.1": (512, 128),
@@ -63,7 +63,9 @@ def test_state_dict_names_and_shapes():
     assert m.gates[0].wg.weight.dtype == torch.float32
     assert float(m.batched_fc1_bias[0].detach().abs().max()) == 0.0
     w = m.batched_fc1_w[0].detach()                                   # trunc_normal(std=0.005), cut at +-2 (absolute)
-    assert 0.004 < float(w.std()) < 0.006 and float(w.abs().max()) < 0.05
+    # (a uniform draw of exactly -1 maps to the lower cut itself, -2: one element in 2^24, so the bulk is checked, not the maximum)
+    bulk = w[w.abs() < 0.05]
+    assert bulk.numel() > 0.9999 * w.numel() and 0.004 < float(bulk.std()) < 0.006 and float(w.abs().max()) <= 2.0
     nb = _readme_module(mlp_fc1_bias=False, mlp_fc2_bias=False)
     assert not any("bias" in k or "_b." in k for k in nb.state_dict())
     assert nb.batched_fc1_bias[0] is None

@@ -69,6 +69,22 @@ extern "C" int hexa_set_option(const char* name, int value) {
 extern "C" const char* hexa_last_error(void) { return g_err; }
 extern "C" int hexa_abi_version(void) { return HEXA_ABI_VERSION; }
 
+// Whether esmm_call, for a slot-summed (m2s) result of these sizes and types, takes the fast path whose slot sum can
+// add one more tensor (`sum_extra`): the same predicate esmm_call applies, for callers that must decide beforehand
+// where that addend is written.
+bool hexa::esmm_slot_sum_takes_extra(const int32_t* route, int w_layout, int T, int k, int in_dim, int out_dim, int E,
+                                     int x_dt, int w_dt, int out_dt, const void* slot_ws) {
+    if (T <= 0 || k <= 1 || !slot_ws || x_dt == HEXA_F32 || !dma_path_enabled()) return false;
+    EsmmArgs a;
+    a.out = nullptr; a.x = nullptr; a.w = nullptr; a.bias = nullptr; a.out_act = nullptr; a.slot_ws = const_cast<void*>(slot_ws);
+    a.r = route_view(route, T, k, E);
+    a.in_dim = in_dim; a.out_dim = out_dim;
+    a.x_per_slot = 1; a.out_per_slot = 0;
+    a.w_layout = w_layout; a.accumulate = 0;
+    a.x_dt = x_dt; a.w_dt = w_dt; a.bias_dt = HEXA_F32; a.out_dt = out_dt; a.act = HEXA_ACT_NONE;
+    return esmm16_dma_supported(a);
+}
+
 // The body of hexa_esmm with one more operand: `sum_extra` (may be null) is a tensor of the result's shape that
 // the slot sum adds on the fast path (m2s, top_k > 1, slot_ws given); *extra_used says whether it was added.
 int hexa::esmm_call(void* out, const void* x, const void* w, const void* bias, const int32_t* route, int m2s,

@@ -295,8 +295,10 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
     if (gate_path) {
         // With several slots on the 16-bit fast path the slot sum of step 10 adds the gate's share as one more
         // addend; otherwise the gate's share is written into dx first and step 10 accumulates onto it.
-        gate_dx_in_ws = dx && k > 1 && d->act_dt != HEXA_F32 && d->w_dt == d->act_dt && dma_path_enabled() &&
-                        (d->hidden % 32) == 0 && (d->d_in % 8) == 0;
+        // (decided with the predicate step 10's call itself applies, so a shape the fast path does not cover --
+        // operands of 4 GiB and more, odd dimensions -- falls back instead of failing)
+        gate_dx_in_ws = dx && esmm_slot_sum_takes_extra(route, HEXA_W_IN_OUT, T, k, d->hidden, d->d_in, E, d->act_dt, d->w_dt,
+                                                        d->act_dt, w.slot_ws);
         if (batching) tg.dwg_reduce = &D;
         RUN(hexa_gate_backward(dx ? (gate_dx_in_ws ? w.dx_gate : dx) : nullptr, dwg, w.dlogits, x, wg, T, d->d_in, E,
                                d->act_dt, w.gate, stream));

@@ -11,6 +11,8 @@
 // Replaces the ESS task of fused_grad_bias_kernel_vectorized_* (kernels/fused_ops_full.cu:372-431).
 #include <algorithm>
 
+#include <mutex>
+
 #include "small_bodies.h"
 
 namespace hexa {
@@ -141,11 +143,13 @@ constexpr int64_t ESS_SCRATCH_FLOATS = HEXA_ESS_NOALLOC_MAX_FLOATS;   // 8 MiB p
 constexpr int ESS_MAX_DEVICES = 64;
 static __device__ __align__(256) float scratch[ESS_SCRATCH_FLOATS];
 static float* g_scratch_ptr[ESS_MAX_DEVICES];
+static std::mutex g_scratch_mutex;   // the first calls of several threads on one device look the address up once
 
 int ess_scratch_for_current_device(float** out) {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= ESS_MAX_DEVICES)
         HEXA_FAIL(HEXA_ERR_LAUNCH, "hexa_ess_noalloc: cannot identify the current device");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (!g_scratch_ptr[dev]) {
         float* ptr = nullptr;
         const hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));

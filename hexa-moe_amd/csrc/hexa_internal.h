@@ -81,6 +81,8 @@ struct EssArgs {
 int esmm_call(void* out, const void* x, const void* w, const void* bias, const int32_t* route, int m2s, int w_layout,
               int accumulate, int T, int k, int in_dim, int out_dim, int E, int x_dt, int w_dt, int bias_dt, int out_dt,
               int act, void* out_act, void* slot_ws, const void* sum_extra, bool* extra_used, void* stream);
+bool esmm_slot_sum_takes_extra(const int32_t* route, int w_layout, int T, int k, int in_dim, int out_dim, int E, int x_dt,
+                               int w_dt, int out_dt, const void* slot_ws);
 int launch_esmm16(const EsmmArgs& a, hipStream_t s);
 int launch_esmm32(const EsmmArgs& a, hipStream_t s);
 // Tuning / testing knobs: 0 = automatic.  Each one starts from an environment variable (read once) and

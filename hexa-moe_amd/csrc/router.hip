@@ -554,6 +554,21 @@ extern "C" int hexa_router_ws_floats(int T, int E, int64_t* out) {
 }
 
 namespace hexa {
+namespace {
+// The LDS tile of the four-lanes-per-token router (with the routing histogram behind it) passes 64 KiB for many
+// experts and a deep top-k: such a launch needs the kernel's dynamic-LDS limit raised first, once per kernel, to the
+// most any supported (E, k) asks for.
+template <typename K> int allow_router_lds(K kernel, size_t bytes) {
+    static bool done = false;   // per kernel
+    if (bytes <= 64 * 1024 || done) return HEXA_OK;
+    constexpr size_t most = sizeof(float) * router4_lds_floats(ROUTER_LDS_E, MAX_TOPK, true);
+    static_assert(most <= 160 * 1024, "LDS of a CU");
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)most) != hipSuccess)
+        HEXA_FAIL(HEXA_ERR_LAUNCH, "router: hipFuncSetAttribute(MaxDynamicSharedMemorySize=%d) failed", (int)most);
+    done = true;
+    return HEXA_OK;
+}
+}  // namespace
 bool router_hist_supported(int E) { return E <= ROUTER_LDS_E; }
 int router_tokens_per_workgroup() { return ROUTER_TB; }
 
@@ -564,10 +579,12 @@ int launch_router_fwd(float* scores, int32_t* idx, const float* logits, const fl
     const int nb = div_up(T, ROUTER_TB);
     float* part_me = ws;
     float* part_cnt = ws + (size_t)nb * E;
-    if (E <= ROUTER_LDS_E)
-        hipLaunchKernelGGL(router_fwd4_kernel, dim3(nb), dim3(ROUTER_TB * ROUTER_G), sizeof(float) * router4_lds_floats(E, k, hist != nullptr),
-                           st, scores, idx, part_me, part_cnt, logits, noise, noise_scale, T, E, k, hist);
-    else
+    if (E <= ROUTER_LDS_E) {
+        const size_t lds = sizeof(float) * router4_lds_floats(E, k, hist != nullptr);
+        if (int rc = allow_router_lds(router_fwd4_kernel, lds)) return rc;
+        hipLaunchKernelGGL(router_fwd4_kernel, dim3(nb), dim3(ROUTER_TB * ROUTER_G), lds, st, scores, idx, part_me, part_cnt, logits,
+                           noise, noise_scale, T, E, k, hist);
+    } else
         hipLaunchKernelGGL(router_fwd_kernel, dim3(nb), dim3(ROUTER_TB), sizeof(float) * 2 * E, st, scores, idx,
                            part_me, part_cnt, logits, noise, noise_scale, T, E, k);
     HEXA_CHECK_LAUNCH("router_fwd");
@@ -586,6 +603,10 @@ int launch_gate_router(float* logits, float* scores, int32_t* idx, const void* x
     float* part_cnt = ws + (size_t)nb * E;
     const size_t lds = sizeof(float) * router4_lds_floats(E, k, hist != nullptr);
     const dim3 grid(nb), block(GATE_ROUTER_NT);
+    if (int rc = x_dt == HEXA_F32    ? allow_router_lds(gate_router_kernel<float>, lds)
+                 : x_dt == HEXA_BF16 ? allow_router_lds(gate_router_kernel<__bf16>, lds)
+                                     : allow_router_lds(gate_router_kernel<_Float16>, lds))
+        return rc;
     if (x_dt == HEXA_F32)
         hipLaunchKernelGGL(gate_router_kernel<float>, grid, block, lds, st, logits, scores, idx, part_me, part_cnt, (const float*)x, wg,
                            noise, noise_scale, T, d, E, k, hist);

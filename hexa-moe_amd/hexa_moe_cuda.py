@@ -44,9 +44,25 @@ def _i32(t, what):
     return t
 
 
+def _forget_routes_of(*written):
+    """Drop the cached routing metadata of every list tensor this call is about to rewrite.  The operators below write
+    through raw device pointers, which does not advance a tensor's version counter, so the cache key alone would not
+    notice a second TOKEN_ASSIGN into the same preallocated lists."""
+    spans = [(t.data_ptr(), t.data_ptr() + t.numel() * t.element_size()) for t in written if t is not None]
+    for key, (_, tok, exp, cum) in list(_route_cache.items()):
+        for held in (tok, exp, cum):
+            if held is None:
+                continue
+            lo, hi = held.data_ptr(), held.data_ptr() + held.numel() * held.element_size()
+            if any(lo < b and a < hi for a, b in spans):
+                del _route_cache[key]
+                break
+
+
 def TOKEN_COUNT(tokens_per_expert, expanded_tokens_per_expert, routings, num_tokens, num_routings):
     _i32(tokens_per_expert, "tokens_per_expert"); _i32(expanded_tokens_per_expert, "expanded_tokens_per_expert")
     _i32(routings, "routings")
+    _forget_routes_of(tokens_per_expert, expanded_tokens_per_expert)
     assert tokens_per_expert.numel() >= num_routings and expanded_tokens_per_expert.numel() >= num_routings + 1
     assert routings.numel() >= num_tokens
     scratch = _scratch(num_tokens, num_routings, routings.device)
@@ -59,6 +75,7 @@ def TOKEN_COUNT(tokens_per_expert, expanded_tokens_per_expert, routings, num_tok
 def TOKEN_ASSIGN(token_idx_list, expert_idx_list, expanded_tokens_per_expert, routings, num_tokens, num_routings):
     _i32(token_idx_list, "token_idx_list"); _i32(expert_idx_list, "expert_idx_list")
     _i32(expanded_tokens_per_expert, "expanded_tokens_per_expert"); _i32(routings, "routings")
+    _forget_routes_of(token_idx_list, expert_idx_list)
     scratch = _scratch(num_tokens, num_routings, routings.device)
     rc = _lib.load().hexa_token_assign(token_idx_list.data_ptr(), expert_idx_list.data_ptr(),
                                        expanded_tokens_per_expert.data_ptr(), routings.data_ptr(), int(num_tokens),
@@ -74,7 +91,8 @@ def _route(token_idx_list, expert_idx_list, num_expanded_tokens, num_tokens, top
     """Routing metadata of the operators for the caller's lists.  The reference's layer calls the matmul ops several
     times per step with the same lists (impls/layers.py:256-274, 409-451); the metadata (and the ESTMM work plan
     that hangs off it) is built once per list contents: the cache key holds the tensors' addresses and version
-    counters, so lists that were rewritten in place are rebuilt."""
+    counters, so lists that were rewritten in place by torch are rebuilt, and TOKEN_COUNT / TOKEN_ASSIGN drop the
+    entries of the tensors they write (_forget_routes_of)."""
     _i32(token_idx_list, "token_idx_list"); _i32(expert_idx_list, "expert_idx_list")
     if token_idx_list.numel() != expert_idx_list.numel():
         raise ValueError("token_idx_list and expert_idx_list differ in length")

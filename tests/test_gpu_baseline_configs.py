@@ -168,3 +168,59 @@ def test_large_token_count(dev):
     assert_close(dw, O.estmm(dy.float(), x.float(), token_ids, offsets, True, E), tol, "estmm")
     db = ops.ess(dy.to(dev), route, True)
     assert_close(db, O.ess(dy.float(), token_ids, offsets, True, E), tol, "ess")
+
+
+def test_benchmark_step_T18432_top2_default_depth_path(dev):
+    """The benchmark's own module and inputs (bench.make_module_and_inputs: T=18432, d=384, h=1536, E=32, top-2,
+    bf16 experts, fp32 gate) through the default path -- one library call per direction -- against the oracle:
+    y, dx and the four parameter gradients of the expert path, then dx and the gate's weight gradient with the
+    auxiliary loss in the backward as the benchmark runs it (the gate's share from fp32 autograd of the oracle's
+    loss on the same routing)."""
+    import bench
+    m, x, dy = bench.make_module_and_inputs(dev)
+    T, k, E = bench.T, bench.K_TOP, bench.E
+    print(f"config benchmark step T={T} d={bench.D} h={bench.H} E={E} k={k} bf16 seed={bench.SEED}", flush=True)
+    tol = TOL[BF16]
+    cpu = lambda t: t.detach().float().cpu()  # noqa: E731
+    W1, W2 = cpu(m.batched_fc1_w[0]), cpu(m.batched_fc2_w[0])
+    b1, b2 = cpu(m.batched_fc1_bias[0]), cpu(m.batched_fc2_bias[0])
+    wg = cpu(m.gates[0].wg.weight)
+    xc, dyc = cpu(x), cpu(dy)
+
+    # expert path alone
+    y, l_aux = m(0, x)
+    routing = m.dispatch_params.routing_.cpu().long()
+    y.backward(dy)
+    torch.cuda.synchronize()
+    logits = xc @ wg.t()
+    scores_ref, routing_ref = O.route_top_k(logits, k)
+    # the expert choice is that of torch.topk on the CPU's fp32 scores, except where two scores tie to within the
+    # rounding of the projection's sums (a handful of tokens in 18432 at most); the oracle below gets the GPU's routing
+    assert int((routing != routing_ref).any(1).sum()) <= 4
+    assert abs(float(l_aux) - float(O.gshard_loss(scores_ref, routing))) < 1e-5
+    y_ref, y1, _ = O.moe_ffn_forward(xc, W1, W2, b1, b2, routing, F.gelu)
+    dx, dW1, dW2, db1, db2 = O.moe_ffn_backward(dyc, xc, y1, W1, W2, True, True, routing, F.gelu)
+    assert_close(y, y_ref, tol, "y")
+    assert_close(x.grad, dx, tol, "dx (expert path)")
+    assert_close(m.batched_fc1_w[0].grad, dW1, tol, "dW1")
+    assert_close(m.batched_fc2_w[0].grad, dW2, tol, "dW2")
+    assert_close(m.batched_fc1_bias[0].grad, db1, tol, "db1")
+    assert_close(m.batched_fc2_bias[0].grad, db2, tol, "db2")
+    assert m.gates[0].wg.weight.grad is None
+
+    # the benchmark's backward: y and the auxiliary loss together (weight 100 so that the gate's share is visible
+    # next to the expert path's in bf16)
+    x.grad = None
+    for p in m.parameters():
+        p.grad = None
+    y, l_aux = m(0, x)
+    torch.autograd.backward([y, l_aux], [dy, torch.full((), 100.0, device=dev)])
+    torch.cuda.synchronize()
+    xg = xc.clone().requires_grad_(True)
+    wgg = wg.clone().requires_grad_(True)
+    loss = O.gshard_loss(torch.softmax(xg @ wgg.t(), 1), routing)
+    gx, gwg = torch.autograd.grad(loss * 100.0, [xg, wgg])
+    assert float(gx.norm()) > 1e-3 * float(dx.norm())
+    assert_close(x.grad, dx + gx, tol, "dx (expert path + gate)")
+    assert_close(m.gates[0].wg.weight.grad, gwg, 1e-4, "dwg")
+    assert_close(m.batched_fc1_w[0].grad, dW1, tol, "dW1 (with l_aux)")

@@ -332,6 +332,35 @@ def _reference_style_ops(dev, pad):
     hexa_moe_cuda.clear_route_cache()
 
 
+def test_token_assign_into_the_same_lists_rebuilds_the_routing_metadata(dev):
+    """A caller that keeps ONE pair of preallocated list tensors (k = 1, so the lists are passed as they are) and
+    refills them with TOKEN_ASSIGN for a new routing: the matmul op behind it must see the new routing.  The
+    operators write through raw pointers, which leaves the tensors' version counters alone."""
+    import hexa_moe_cuda
+    hexa_moe_cuda.clear_route_cache()
+    T, d_in, d_out, E = 512, 64, 128, 4
+    x, W, b = make_linear(T, d_in, d_out, E, 1, seed=31, dtype=F32, m2s=False)
+    tok = torch.empty(T, dtype=torch.int32, device=dev)
+    exp = torch.empty(T, dtype=torch.int32, device=dev)
+    tpe = torch.zeros(E, dtype=torch.int32, device=dev)
+    expd = torch.zeros(E + 1, dtype=torch.int32, device=dev)
+    cum = torch.tensor([0, T], dtype=torch.int32, device=dev)
+    for seed in (41, 42, 43):
+        routing = make_routing(T, E, 1, seed=seed).to(torch.int32)
+        _, offsets, token_ids = O.route_build(routing, E)
+        want = O.esmm(x.double(), W.double(), b.double(), token_ids, offsets, False)
+        col = routing[:, 0].contiguous().to(dev)
+        hexa_moe_cuda.TOKEN_COUNT(tpe, expd, col, T, E)
+        hexa_moe_cuda.TOKEN_ASSIGN(tok, exp, expd, col, T, E)       # same tensors every time, no torch op in between
+        hid = torch.zeros(1, T, d_out, dtype=F32, device=dev)
+        hexa_moe_cuda.ESMM_TENSOR_CORE(hid.reshape(-1), x.to(dev).reshape(-1), W.to(dev).reshape(-1), b.to(dev).reshape(-1),
+                                       tok, exp, cum, True, True, True, False, T, 1, d_in, d_out, E)
+        torch.cuda.synchronize()
+        assert_close(hid, want, 1e-5, f"ESMM_TENSOR_CORE after re-assignment, seed {seed}")
+        assert len(hexa_moe_cuda._route_cache) == 1
+    hexa_moe_cuda.clear_route_cache()
+
+
 def test_cpu_tensors_are_rejected(dev):
     from hexa_moe import ops
     with pytest.raises(RuntimeError, match="GPU only"):

@@ -79,3 +79,27 @@ def test_noalloc_rejects_sizes_beyond_the_builtin_scratch(dev):
     rc = lib.hexa_ess_noalloc(db.data_ptr(), dy.data_ptr(), route.blob.data_ptr(), 0, 0, T, 1, d_out, E, 0, 0,
                               torch.cuda.current_stream().cuda_stream)
     assert rc == -2 and b"built-in scratch" in lib.hexa_last_error()
+
+
+def test_noalloc_allocates_nothing(dev):
+    """The property the entry point exists for: after a warm call, further calls leave the device's free memory
+    as it was (hipMemGetInfo through torch: neither the library nor the runtime took or returned a byte)."""
+    from hexa_moe import _lib, ops
+    lib = _lib.load()
+    T, d_out, E, k = 9000, 264, 8, 2
+    routing = make_routing(T, E, k, seed=341, skew="zipf")
+    route = ops.route_build(routing.to(dev), E)
+    dy = torch.randn(k, T, d_out, device=dev, dtype=torch.bfloat16)
+    db = torch.zeros(E, d_out, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    call = lambda: lib.hexa_ess_noalloc(db.data_ptr(), dy.data_ptr(), route.blob.data_ptr(), 1, 0, T, k, d_out, E,  # noqa: E731
+                                        DT[torch.bfloat16], 0, st)
+    assert call() == 0
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    reserved0 = torch.cuda.memory_reserved()
+    for _ in range(5):
+        assert call() == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0 and torch.cuda.memory_reserved() == reserved0

@@ -175,18 +175,48 @@ template <typename TC> __device__ __forceinline__ float lo16(unsigned w) { retur
 template <typename TC> __device__ __forceinline__ float hi16(unsigned w) { return from_bits16<TC>(w >> 16); }
 
 // GELU and GELU' of a value that has been rounded to bf16 are functions of 16 bits.  The store wavefronts look them up
-// in a table the workgroup builds at its start instead of evaluating them: every magnitude from 2^-14 up to (not
-// including) 8, both signs -- LUT_R entries per sign, the polynomial's own results (so nothing changes in any bit),
-// as bf16 for GELU and as fp32 for GELU' (which is multiplied before rounding).  A piece with a value outside that
-// range (zeros, |x| >= 8, NaN) takes the polynomial: one wavefront-wide branch per 16-byte piece.  The fused
-// epilogues are bound by their vector instructions (about 18 and 31 per element): a lookup is 6.
-constexpr unsigned LUT_M_LO = 0x3880, LUT_M_HI = 0x4100, LUT_R = LUT_M_HI - LUT_M_LO;
-template <typename TC, int ACT> constexpr int pipe_lut_bytes() {
-    return !std::is_same<TC, __bf16>::value ? 0 : ACT == HEXA_ACT_GELU ? 2 * LUT_R * 2 : ACT == HEXA_ACT_GELU_BWD ? 2 * LUT_R * 4 : 0;
+// in a table the workgroup builds at its start instead of evaluating them: every magnitude from LUT_M_LO (2^-17, or
+// 2^-14 where LDS is short) up to (not including) 8, both signs, the polynomial's own results (so nothing changes in
+// any bit), as bf16 for GELU and as fp32 for GELU' (which is multiplied before rounding).  Entry 2 * (magnitude bits
+// - LUT_M_LO) + sign: the two 16-bit values of a 32-bit word are turned into two table addresses with packed 16-bit
+// arithmetic (four vector instructions per element instead of nine).  A piece with a value outside that range
+// (zeros, |x| >= 8, NaN) takes the polynomial: one wavefront-wide branch per 16-byte piece.  The fused epilogues are
+// bound by their vector instructions.
+constexpr unsigned LUT_M_HI = 0x4100;
+template <typename TC, int ACT, bool COLSUM> constexpr unsigned pipe_lut_lo() {
+    // GELU' with column sums: fp32 entries next to the column-sum area leave room for magnitudes from 2^-14 only
+    return ACT == HEXA_ACT_GELU_BWD && COLSUM ? 0x3880u : 0x3700u;
 }
-__device__ __forceinline__ unsigned lds_read_u16_async(unsigned addr) {
+template <typename TC, int ACT, bool COLSUM> constexpr int pipe_lut_bytes() {
+    constexpr int r = (int)(LUT_M_HI - pipe_lut_lo<TC, ACT, COLSUM>());
+    return !std::is_same<TC, __bf16>::value ? 0 : ACT == HEXA_ACT_GELU ? 2 * r * 2 : ACT == HEXA_ACT_GELU_BWD ? 2 * r * 4 : 0;
+}
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u16x2 as_u16x2(unsigned w) {
+    union { unsigned u; u16x2 v; } c;
+    c.u = w;
+    return c.v;
+}
+__device__ __forceinline__ unsigned as_u32(u16x2 v) {
+    union { unsigned u; u16x2 v; } c;
+    c.v = v;
+    return c.u;
+}
+// The table positions (as byte offsets, entries of 1 << SH bytes) of the two 16-bit values of w, packed in one word;
+// `far` collects the largest distance from the table's first magnitude (a magnitude below it wraps to a huge
+// one), so far >= the table's length says some value is outside.
+template <unsigned LO, int SH> __device__ __forceinline__ unsigned lut_offsets(unsigned w, u16x2& far) {
+    const u16x2 lo2 = {(unsigned short)LO, (unsigned short)LO};
+    const u16x2 u = as_u16x2(w & 0x7fff7fffu) - lo2;
+    far = __builtin_elementwise_max(far, u);
+    const u16x2 sh = {(unsigned short)(SH + 1), (unsigned short)(SH + 1)};
+    return as_u32(u << sh) | ((w >> (15 - SH)) & ((1u << SH) * 0x00010001u));
+}
+// (the 16-bit LDS loads that target one half of a register clear the other half on this chip, so two entries
+// are read into two registers and joined with one shift-or)
+template <int OFF> __device__ __forceinline__ unsigned lds_read_u16_async(unsigned addr) {
     unsigned r;
-    asm volatile("ds_read_u16 %0, %1" : "=v"(r) : "v"(addr));
+    asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
     return r;
 }
 
@@ -201,20 +231,23 @@ struct PipeK {
 #endif
 constexpr int PIPE_COPY_WAVES = PIPE_CW, PIPE_STORE_WAVES = PIPE_SW;
 
-// LUT: bytes of the activation table behind everything else (0 = none)
-template <typename C, int LUT = 0> struct PipeLds {
+// LUT: bytes of the activation table (0 = none).  The table comes first: its entries are addressed with 16-bit
+// offsets from the start of the workgroup's LDS.
+template <typename C, int LUT = 0, bool COLSUM = true> struct PipeLds {
     static constexpr int CP = C::BN * 2 + 16;                 // pitch of a staged 16-bit result row
-    static constexpr int STAGING_AT = C::STAGE_AREA;
+    static constexpr int LUT_AT = 0;
+    static constexpr int STAGES_AT = (LUT + 1023) / 1024 * 1024;
+    static constexpr int STAGING_AT = STAGES_AT + C::STAGE_AREA;
     static constexpr int TOK_AT = STAGING_AT + C::BM * CP;    // 3 x BM token ids
     static constexpr int BIAS_SLOT = 1024;                    // one wavefront copy (64 lanes x 16 bytes) per slot
     static constexpr int BIAS_AT = TOK_AT + 3 * C::BM * 4;    // 3 slots of raw bias elements (BN x 4 bytes used at most)
     static constexpr int INFO_AT = BIAS_AT + 3 * BIAS_SLOT;   // PIPE_MAX_ROUNDS x int4
     static constexpr int RED_AT = INFO_AT + PIPE_MAX_ROUNDS * 16;   // column-sum partials: store wavefronts x BN floats
-    static constexpr int SINK_AT = RED_AT + PIPE_STORE_WAVES * C::BN * 4;    // 256 bytes nobody reads (filler copies)
-    static constexpr int LUT_AT = SINK_AT + 256;
-    static constexpr int BYTES = LUT_AT + LUT;
+    static constexpr int SINK_AT = RED_AT + (COLSUM ? PIPE_STORE_WAVES * C::BN * 4 : 0);    // 256 bytes nobody reads (filler copies)
+    static constexpr int BYTES = SINK_AT + 256;
     static_assert(BYTES <= 160 * 1024, "LDS of a CU");
     static_assert(C::BN * 4 <= BIAS_SLOT, "bias slot");
+    static_assert(LUT < 65536, "table offsets are 16 bits");
 };
 
 // ACT: HEXA_ACT_NONE / _GELU / _GELU_BWD.  COLSUM: also per-tile column sums of the stored result.
@@ -226,8 +259,9 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
     constexpr int R_CPW = C::R_COPIES / CW, F_CPW = C::F_COPIES / CW, CPW = R_CPW + F_CPW;   // copies per copy wavefront and stage
     static_assert(C::R_COPIES % CW == 0 && C::F_COPIES % CW == 0, "copies must divide evenly over the copy wavefronts");
     static_assert(BM <= 64 * CW, "at most one 64-id copy per copy wavefront");
-    constexpr int LUT = pipe_lut_bytes<TC, ACT>();
-    using L = PipeLds<C, LUT>;
+    constexpr int LUT = pipe_lut_bytes<TC, ACT, COLSUM>();
+    constexpr unsigned LUT_LO = pipe_lut_lo<TC, ACT, COLSUM>(), LUT_R = LUT_M_HI - LUT_LO;
+    using L = PipeLds<C, LUT, COLSUM>;
     constexpr int CP = L::CP;
     constexpr int LPR = BN / 8;                         // 16-byte pieces per staged row
     constexpr int PIECES = BM * LPR / NTS;              // pieces per store lane and tile
@@ -267,10 +301,10 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
         sInfo[i] = make_int4(rec.x, rec.y, rec.z | ((mtg - cum[sl]) << 10), (s << 24) | nt);
     }
     if constexpr (LUT > 0) {
-        // entry sign * LUT_R + (magnitude bits - LUT_M_LO): what the polynomial gives for exactly that bf16 value
+        // entry 2 * (magnitude bits - LUT_LO) + sign: what the polynomial gives for exactly that bf16 value
         for (unsigned i = tid; i < 2 * LUT_R; i += NT_ALL) {
-            const unsigned sign = i >= LUT_R ? 1u : 0u;
-            const float xv = from_bits16<TC>((unsigned short)((sign << 15) | (LUT_M_LO + i - sign * LUT_R)));
+            const unsigned sign = i & 1u;
+            const float xv = from_bits16<TC>((unsigned short)((sign << 15) | (LUT_LO + (i >> 1))));
             if (ACT == HEXA_ACT_GELU) reinterpret_cast<unsigned short*>(smem + L::LUT_AT)[i] = (unsigned short)(pack2<TC>(gelu_poly(xv), 0.f) & 0xffff);
             else reinterpret_cast<float*>(smem + L::LUT_AT)[i] = gelu_grad_poly(xv);
         }
@@ -301,7 +335,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
         for (int r = 0; r < ntiles; ++r) {
             for (int kt = 0; kt < nk; ++kt) {
                 barrier_nofence();                       // the copies of this step have landed
-                const unsigned base = lds0 + stage * C::STAGE_BYTES;
+                const unsigned base = lds0 + L::STAGES_AT + stage * C::STAGE_BYTES;
                 mma_stage_ahead<TC, C, W_IN_OUT>(base, base + C::R_BYTES, wr, wf, lane, acc);
                 stage = stage + 1 == STAGES ? 0 : stage + 1;
             }
@@ -409,7 +443,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
             }
         };
         auto issue = [&](int stage) {
-            char* base = smem + stage * C::STAGE_BYTES;
+            char* base = smem + L::STAGES_AT + stage * C::STAGE_BYTES;
 #pragma unroll
             for (int i = 0; i < R_CPW; ++i) {
                 dma16(xbase + (size_t)srcR[i], base + (cw + CW * i) * 1024);
@@ -516,16 +550,17 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
     // earlier pieces (a store is skipped when no lane of the wavefront has a valid row, so their number is not
     // fixed): allowing PIECES-1-q outstanding operations waits for that load in every case.
     const unsigned stg_lane = lds0 + L::STAGING_AT + rl0 * CP + c * 16;
-    // table positions of the eight 16-bit values of a piece; `far` = the largest distance from the table's first
-    // magnitude (unsigned: a magnitude below it wraps to a huge one), so far >= LUT_R says some value is outside
-    auto lut_index = [&](const unsigned (&w)[4], unsigned (&idx)[8], unsigned& far) {
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const unsigned tl = (w[u] & 0x7fffu) - LUT_M_LO, th = ((w[u] >> 16) & 0x7fffu) - LUT_M_LO;
-            far = max(far, max(tl, th));
-            idx[2 * u] = tl + ((w[u] >> 15) & 1u) * LUT_R;
-            idx[2 * u + 1] = th + (w[u] >> 31) * LUT_R;
-        }
+    // with the table at the very start of the workgroup's LDS its 16-bit offsets are LDS addresses
+    const bool lut_ok = LUT > 0 && lds0 == 0;
+    // rows are addressed as (row * 2N + column) in 32 bits; a 24-bit multiply when both factors allow
+    const bool mul24 = (size_t)p.T * 8 < ((size_t)1 << 24) && N < (1 << 22);
+    const unsigned pitch = (unsigned)N * 2u;
+    auto row_offset = [&](const auto& t, int tok) {
+        const unsigned row = (unsigned)t.out_base + (unsigned)tok;
+        return (mul24 ? __umul24(row, pitch) : row * pitch) + (unsigned)t.n * 2u;
+    };
+    auto in_table = [&](u16x2 far) {
+        return lut_ok && __builtin_amdgcn_ballot_w64(max(far.x, far.y) >= (unsigned short)LUT_R) == 0;
     };
     auto piece = [&](const TileCtx& t, auto qc, u32x4 y1v) {
         constexpr int q = decltype(qc)::value;
@@ -542,19 +577,24 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
         const bool ok = rl < t.rows && t.col_ok;
         if (!ok) return;
         // results, too, are addressed as a base every lane shares plus a 32-bit byte offset
-        const unsigned boff = (unsigned)(((t.out_base + tok) * N + t.n) * 2);
+        const unsigned boff = row_offset(t, tok);
         char* const outb = reinterpret_cast<char*>(t.to_ws ? p.ws : p.out);
         unsigned vw[4] = {val.x, val.y, val.z, val.w};
         if (ACT == HEXA_ACT_GELU_BWD) {
             const unsigned yw[4] = {y1v.x, y1v.y, y1v.z, y1v.w};
             bool looked_up = false;
             if constexpr (LUT > 0) {
-                unsigned idx[8], far = 0;
-                lut_index(yw, idx, far);
-                if (__builtin_amdgcn_ballot_w64(far >= LUT_R) == 0) {   // every value of the wavefront's pieces is in the table
+                unsigned at[4];
+                u16x2 far = {0, 0};
+#pragma unroll
+                for (int u = 0; u < 4; ++u) at[u] = lut_offsets<LUT_LO, 2>(yw[u], far);
+                if (in_table(far)) {   // every value of the wavefront's pieces is in the table
                     unsigned g[8];
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) g[j] = lds_read_i32(lds0 + L::LUT_AT + idx[j] * 4);
+                    for (int u = 0; u < 4; ++u) {
+                        g[2 * u] = (unsigned)lds_read32_async<L::LUT_AT>(at[u] & 0xffffu);
+                        g[2 * u + 1] = (unsigned)lds_read32_async<L::LUT_AT>(at[u] >> 16);
+                    }
                     lds_wait();
 #pragma unroll
                     for (int j = 0; j < 8; ++j) asm volatile("" : "+v"(g[j]));
@@ -576,15 +616,20 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
             for (int u = 0; u < 4; ++u) { cs[2 * u] += lo16<TC>(vw[u]); cs[2 * u + 1] += hi16<TC>(vw[u]); }
         }
         if (ACT == HEXA_ACT_GELU) {   // applied to the value as stored (rounded), like act(y1) on the tensor
-            unsigned aw[4];
+            unsigned aw[4] = {0u, 0u, 0u, 0u};
             bool looked_up = false;
             if constexpr (LUT > 0) {
-                unsigned idx[8], far = 0;
-                lut_index(vw, idx, far);
-                if (__builtin_amdgcn_ballot_w64(far >= LUT_R) == 0) {
+                unsigned at[4];
+                u16x2 far = {0, 0};
+#pragma unroll
+                for (int u = 0; u < 4; ++u) at[u] = lut_offsets<LUT_LO, 1>(vw[u], far);
+                if (in_table(far)) {
                     unsigned g[8];
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) g[j] = lds_read_u16_async(lds0 + L::LUT_AT + idx[j] * 2);
+                    for (int u = 0; u < 4; ++u) {
+                        g[2 * u] = lds_read_u16_async<L::LUT_AT>(at[u] & 0xffffu);
+                        g[2 * u + 1] = lds_read_u16_async<L::LUT_AT>(at[u] >> 16);
+                    }
                     lds_wait();
 #pragma unroll
                     for (int j = 0; j < 8; ++j) asm volatile("" : "+v"(g[j]));
@@ -611,7 +656,7 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
         for (int q = 0; q < PIECES; ++q) {
             asm volatile("" : "+v"(tok[q]));
             const bool ok = rl0 + q * PROWS < t.rows && t.col_ok;
-            y[q] = global_load128_async(p.out_act, ok ? (unsigned)(((t.out_base + tok[q]) * N + t.n) * 2) : 0u);
+            y[q] = global_load128_async(p.out_act, ok ? row_offset(t, tok[q]) : 0u);
         }
     };
     // column sums of the tile just stored: the lanes of a wavefront that hold the same piece, then (after the
@@ -685,7 +730,7 @@ template <typename TC, bool IO, int ACT, bool COLSUM>
 int launch_pipe_t(PipeK& pk, int grid, hipStream_t st) {
     using C = CfgP;
     auto kernel = esmm16_pipe_kernel<TC, IO, ACT, COLSUM, C>;
-    constexpr int bytes = PipeLds<C, pipe_lut_bytes<TC, ACT>()>::BYTES;
+    constexpr int bytes = PipeLds<C, pipe_lut_bytes<TC, ACT, COLSUM>(), COLSUM>::BYTES;
     if (int rc = ensure_smem(kernel, bytes)) return rc;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)), bytes, st, pk);
     HEXA_CHECK_LAUNCH("esmm16_pipe");

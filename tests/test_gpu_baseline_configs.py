@@ -208,19 +208,19 @@ def test_benchmark_step_T18432_top2_default_depth_path(dev):
     assert_close(m.batched_fc2_bias[0].grad, db2, tol, "db2")
     assert m.gates[0].wg.weight.grad is None
 
-    # the benchmark's backward: y and the auxiliary loss together (weight 100 so that the gate's share is visible
+    # the benchmark's backward: y and the auxiliary loss together (weight 2e4 so that the gate's share is visible
     # next to the expert path's in bf16)
     x.grad = None
     for p in m.parameters():
         p.grad = None
     y, l_aux = m(0, x)
-    torch.autograd.backward([y, l_aux], [dy, torch.full((), 100.0, device=dev)])
+    torch.autograd.backward([y, l_aux], [dy, torch.full((), 2e4, device=dev)])
     torch.cuda.synchronize()
     xg = xc.clone().requires_grad_(True)
     wgg = wg.clone().requires_grad_(True)
     loss = O.gshard_loss(torch.softmax(xg @ wgg.t(), 1), routing)
-    gx, gwg = torch.autograd.grad(loss * 100.0, [xg, wgg])
-    assert float(gx.norm()) > 1e-3 * float(dx.norm())
+    gx, gwg = torch.autograd.grad(loss * 2e4, [xg, wgg])
+    assert float(gx.norm()) > 3e-2 * float(dx.norm())
     assert_close(x.grad, dx + gx, tol, "dx (expert path + gate)")
     assert_close(m.gates[0].wg.weight.grad, gwg, 1e-4, "dwg")
     assert_close(m.batched_fc1_w[0].grad, dW1, tol, "dW1 (with l_aux)")

@@ -27,6 +27,7 @@ OptEntry g_opts[OPT_COUNT] = {
     {"batch", "HEXA_MOE_BATCH", 0, false},
     {"ffn_fused", "HEXA_MOE_FFN_FUSED", 0, false},
     {"gate_router", "HEXA_MOE_GATE_ROUTER", 0, false},
+    {"estmm_pipe", "HEXA_ESTMM_PIPE", 0, false},
 };
 }  // namespace
 
@@ -142,7 +143,7 @@ extern "C" int hexa_esmm(void* out, const void* x, const void* w, const void* bi
 
 extern "C" int hexa_estmm(void* dw, const void* dy, const void* x, const int32_t* route, int dy_per_slot,
                           int x_per_slot, int accumulate, int T, int k, int out_dim, int in_dim, int E, int dt,
-                          int dw_dt, const int32_t* plan, int max_slots, float* scratch, void* stream) {
+                          int dw_dt, int32_t* plan, int max_slots, float* scratch, void* stream) {
     if (int rc = check_sizes("hexa_estmm", T, k, E, in_dim, out_dim)) return rc;
     if (!dw || !route || !dy || !x) HEXA_FAIL(HEXA_ERR_ARG, "hexa_estmm: null pointer");
     if (!is_dt(dt) || !is_dt(dw_dt)) HEXA_FAIL(HEXA_ERR_ARG, "hexa_estmm: unknown element type");
@@ -155,17 +156,22 @@ extern "C" int hexa_estmm(void* dw, const void* dy, const void* x, const int32_t
     a.m_dim = out_dim; a.n_dim = in_dim;
     a.p_per_slot = dy_per_slot ? 1 : 0; a.q_per_slot = x_per_slot ? 1 : 0;
     a.accumulate = accumulate ? 1 : 0; a.pq_dt = dt; a.dw_dt = dw_dt;
-    a.plan = (plan && scratch && max_slots >= 2) ? plan : nullptr;
-    a.max_slots = a.plan ? max_slots : 0;
-    a.scratch = a.plan ? scratch : nullptr;
+    // a plan without scratch (max_slots < 2) cuts no expert: it orders the work and carries the persistent kernel's queue
+    a.plan = plan;
+    a.max_slots = (plan && scratch && max_slots >= 2) ? max_slots : 0;
+    a.scratch = a.max_slots ? scratch : nullptr;
+    if (is_16(dt) && dma_path_enabled() && estmm_pipe_wanted(a.r) && estmm16_pipe_supported(a)) return launch_estmm16_pipe(a, st);
+    if (!a.max_slots) a.plan = nullptr;
     if (is_16(dt) && dma_path_enabled() && estmm16_dma_supported(a)) return launch_estmm16_dma(a, st);
     return is_16(dt) ? launch_estmm16(a, st) : launch_estmm32(a, st);
 }
 
-extern "C" int hexa_estmm_plan(int32_t* plan, const int32_t* route, int T, int k, int E, int max_slots, void* stream) {
+extern "C" int hexa_estmm_plan(int32_t* plan, const int32_t* route, int T, int k, int E, int max_slots, int out_dim,
+                               int in_dim, void* stream) {
     if (int rc = check_sizes("hexa_estmm_plan", T, k, E, 8, 8)) return rc;
-    if (!plan || !route || max_slots < 0) HEXA_FAIL(HEXA_ERR_ARG, "hexa_estmm_plan: bad arguments");
-    return launch_estmm_plan(plan, route_view(route, T, k, E), max_slots, (hipStream_t)stream);
+    if (!plan || !route || max_slots < 0 || out_dim < 0 || in_dim < 0) HEXA_FAIL(HEXA_ERR_ARG, "hexa_estmm_plan: bad arguments");
+    const RouteView r = route_view(route, T, k, E);
+    return launch_estmm_plan(plan, r, max_slots, estmm_plan_cap_for(r, out_dim, in_dim), (hipStream_t)stream);
 }
 
 extern "C" int hexa_ess(void* db, const void* dy, const int32_t* route, int dy_per_slot, int accumulate, int T, int k,
@@ -200,7 +206,7 @@ extern "C" int hexa_ess_noalloc(void* db, const void* dy, const int32_t* route, 
 extern "C" int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y, const void* w, const void* x,
                                const int32_t* route, int m2s, int accumulate, int T, int k, int in_dim, int out_dim,
                                int E, int act_dt, int w_dt, int jx_dt, int jw_dt, int jb_dt, void* slot_ws,
-                               const int32_t* plan, int max_slots, float* estmm_scratch, float* ess_ws,
+                               int32_t* plan, int max_slots, float* estmm_scratch, float* ess_ws,
                                int64_t ess_ws_floats, void* stream) {
     if (!j_x || !j_w || !j_y || !w || !x || !route) HEXA_FAIL(HEXA_ERR_ARG, "hexa_fused_grad: null pointer");
     // ESMM task: j_x = j_y . w[e] with w [E][out][in] read as an [E][in'=out][out'=in] weight; the

@@ -70,7 +70,7 @@ int carve_backward(const hexa_moe_depth_desc& d, void* ws, BwdWs* out) {
     // one plan and one scratch area serve both ESTMM calls (they run one after the other on the stream)
     const int s2 = estmm_slots(d, d.hidden, d.d_out), s1 = estmm_slots(d, d.hidden, d.d_in);
     out->slots = std::min(s1, s2);
-    out->plan = static_cast<int32_t*>(c.take((int64_t)(4 * E + 1) * 4));
+    out->plan = static_cast<int32_t*>(c.take((int64_t)HEXA_ESTMM_PLAN_INTS(E) * 4));
     out->estmm = out->slots >= 2
                      ? static_cast<float*>(c.take((int64_t)out->slots * d.hidden * std::max(d.d_in, d.d_out) * 4))
                      : nullptr;
@@ -145,8 +145,10 @@ extern "C" int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* 
     const int T = d->num_tokens, k = d->top_k, E = d->num_experts;
     const EventPairs ev{events, num_events, (hipStream_t)stream};
     // the work plan of the backward's ESTMM calls depends on the routing only: made here when the caller keeps it
+    // (without scratch slots it cuts no expert, but still orders the work and carries the persistent kernel's queue)
     const int plan_slots = std::min(estmm_slots(*d, d->hidden, d->d_out), estmm_slots(*d, d->hidden, d->d_in));
-    if (plan && plan_slots < 2) plan = nullptr;
+    if (plan && d->act_dt == HEXA_F32) plan = nullptr;
+    const int plan_cap = estmm_plan_cap_for(route_view(route, T, k, E), d->hidden, std::min(d->d_in, d->d_out));
     bool routed = false;
     if (wg) {
         if (!logits || !scores || !stats || (d->loss == 1 && !thr)) HEXA_FAIL(HEXA_ERR_ARG, "%s: null router state", who);
@@ -165,7 +167,7 @@ extern "C" int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* 
             else
                 RUN(launch_router_fwd(scores, idx, logits, noise, d->noise_scale, T, E, k, w.router, w.hist, (hipStream_t)stream));
             RUN(launch_route_from_hist(idx, T, k, E, route, w.hist, router_tokens_per_workgroup(), stats + 2 * E, stats,
-                                       stats + E, w.router, plan, plan_slots, (hipStream_t)stream));
+                                       stats + E, w.router, plan, plan_slots, plan_cap, (hipStream_t)stream));
             routed = true;
         } else if (d->loss == 0) {
             RUN(hexa_router_forward(scores, idx, stats, stats + E, stats + 2 * E, logits, noise, d->noise_scale, T, E, k,
@@ -178,7 +180,7 @@ extern "C" int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* 
     }
     if (!routed) {
         RUN(hexa_route_build(idx, 0, k, 1, T, k, E, route, stream));
-        if (plan) RUN(hexa_estmm_plan(plan, route, T, k, E, plan_slots, stream));
+        if (plan) RUN(launch_estmm_plan(plan, route_view(route, T, k, E), plan_slots, plan_cap, (hipStream_t)stream));
     }
     if (option(OPT_FFN_FUSED) == 1 && dma_path_enabled() &&
         ffn16_fused_supported(T, k, d->d_in, d->hidden, d->d_out, d->act_dt, d->w_dt, d->b1_dt, d->b2_dt)) {
@@ -205,7 +207,7 @@ extern "C" int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* 
 extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void* dy, const float* grad_l_aux,
                                        const void* x, const float* wg, const void* fc1_w, const void* fc2_w,
                                        const float* scores, const int32_t* idx, const float* thr, const float* stats,
-                                       const int32_t* route, const int32_t* plan, const void* y1, const void* y2,
+                                       const int32_t* route, int32_t* plan, const void* y1, const void* y2,
                                        void* dx, float* dwg, void* dw1, void* db1, void* dw2, void* db2, void* dy1,
                                        void* ws, int64_t ws_bytes, void* const* events, int num_events, void* stream) {
     const char* who = "hexa_moe_depth_backward";
@@ -255,15 +257,17 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
         tg = DeferTargets();
     }
     RUN(batch_flush(A, st));
-    const bool planned = w.slots >= 2 && (dw1 || dw2);
-    if (planned && !plan) RUN(hexa_estmm_plan(w.plan, route, T, k, E, w.slots, stream));
-    if (planned && plan) w.plan = const_cast<int32_t*>(plan);   // made by the forward for the same routing and slot count
+    const bool planned = d->act_dt != HEXA_F32 && (dw1 || dw2);
+    if (planned && !plan)
+        RUN(launch_estmm_plan(w.plan, route_view(route, T, k, E), w.slots,
+                              estmm_plan_cap_for(route_view(route, T, k, E), d->hidden, std::min(d->d_in, d->d_out)), st));
+    if (planned && plan) w.plan = plan;   // made by the forward for the same routing and slot count
     // step 5: dW2 = ESTMM(act(y1), dy): the per-slot operand supplies the rows of dW2 [E][hidden][d_out]
     if (dw2) {
         if (batching) tg.fixup = &B;
         RUN(ev.begin(2));
         RUN(hexa_estmm(dw2, y2, dy, route, 1, 0, 0, T, k, d->hidden, d->d_out, E, d->act_dt, d->gw2_dt,
-                       planned ? w.plan : nullptr, planned ? w.slots : 0, planned ? w.estmm : nullptr, stream));
+                       planned ? w.plan : nullptr, planned ? w.slots : 0, planned && w.slots >= 2 ? w.estmm : nullptr, stream));
         RUN(ev.end(2));
         tg = DeferTargets();
     }
@@ -285,7 +289,7 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
             if (batching) tg.fixup = &C;
             RUN(ev.begin(3));
             RUN(hexa_estmm(dw1, dy1, x, route, 1, 0, 0, T, k, d->hidden, d->d_in, E, d->act_dt, d->gw1_dt,
-                           planned ? w.plan : nullptr, planned ? w.slots : 0, planned ? w.estmm : nullptr, stream));
+                           planned ? w.plan : nullptr, planned ? w.slots : 0, planned && w.slots >= 2 ? w.estmm : nullptr, stream));
             RUN(ev.end(3));
             tg = DeferTargets();
         }

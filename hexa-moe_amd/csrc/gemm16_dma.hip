@@ -654,15 +654,7 @@ int launch_estmm_dma_c(const EstmmArgs& a, hipStream_t st) {
     if (a.pq_dt == HEXA_BF16) rc = o32 ? launch_estmm_dma_t<__bf16, true, C>(p, grid, st) : launch_estmm_dma_t<__bf16, false, C>(p, grid, st);
     else rc = o32 ? launch_estmm_dma_t<_Float16, true, C>(p, grid, st) : launch_estmm_dma_t<_Float16, false, C>(p, grid, st);
     if (rc || !p.plan) return rc;
-    SmallTask t;
-    t.kind = TASK_FIXUP;
-    t.fixup = FixupK{a.dw, p.plan, p.scratch, E, mn, a.dw_dt, a.accumulate, (int)((mn / 4 + 255) / 256)};
-    t.blocks = t.fixup.gx * E;
-    if (!defer_task(defer_targets().fixup, t)) {
-        hipLaunchKernelGGL(estmm_fixup_kernel, dim3(t.blocks), dim3(256), 0, st, t.fixup);
-        HEXA_CHECK_LAUNCH("estmm_fixup");
-    }
-    return HEXA_OK;
+    return launch_estmm_fixup(a, st);
 }
 
 template <typename C>
@@ -736,10 +728,50 @@ int launch_colsum_fold(const EsmmArgs& a, int mt_ub, int tile_rows, int ntn, int
     return HEXA_OK;
 }
 
-int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, hipStream_t st) {
+// the task that adds the parts of the experts a plan has cut (a launch of its own unless a batch takes it)
+int launch_estmm_fixup(const EstmmArgs& a, hipStream_t st) {
+    const long mn = (long)a.m_dim * a.n_dim;
+    SmallTask t;
+    t.kind = TASK_FIXUP;
+    t.fixup = FixupK{a.dw, a.plan, a.scratch, a.r.E, mn, a.dw_dt, a.accumulate, (int)((mn / 4 + 255) / 256)};
+    t.blocks = t.fixup.gx * a.r.E;
+    if (!defer_task(defer_targets().fixup, t)) {
+        hipLaunchKernelGGL(estmm_fixup_kernel, dim3(t.blocks), dim3(256), 0, st, t.fixup);
+        HEXA_CHECK_LAUNCH("estmm_fixup");
+    }
+    return HEXA_OK;
+}
+
+// The persistent kernel (one workgroup per CU, an item at a time at the CU's full rate) against the one-item-per-
+// workgroup kernel (four workgroups per CU).  Alone, with its operands in the memory-side cache, the persistent kernel
+// is the faster one (73 against 80 us + fix-up at 1152 rows per expert) and needs no fp32 partial results; inside a
+// layer's backward, where every operand row comes from HBM, its two stages of copies in flight per CU (64 KB) do
+// not cover the memory latency (a step waits 1900 instead of 1100 cycles for its rows) and it takes 86-89 us against
+// 81-85, and with an item only one or two steps long its per-item cost loses outright (0.41 against 0.37 ms per
+// layer at 72 rows per expert).  So it runs on request only (option "estmm_pipe" = 1).
+bool estmm_pipe_wanted(const RouteView& r) {
+    (void)r;
+    return option(OPT_ESTMM_PIPE) == 1 && option(OPT_TILE) == 0;   // (a forced tile shape selects the one-item-per-workgroup kernels)
+}
+
+// Rows above which an expert's list is cut into parts (out_dim, in_dim = 0: unknown result size).  Both kernels hand
+// their items out longest-first (the hardware's workgroup dispatcher does it for the one-item-per-workgroup kernel), so a
+// cut only pays when one item would be longer than a workgroup slot's share of the launch: rows of all lists x blocks
+// per expert / slots -- 256 for the persistent kernel, 1024 (four workgroups per CU, each at a quarter of the CU's
+// rate) and never less than 1.5x the mean load for the other.
+int estmm_plan_cap_for(const RouteView& r, int out_dim, int in_dim) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8)
+        cus = 256;
+    const int tiles = (out_dim > 0 && in_dim > 0) ? div_up(out_dim, 128) * div_up(in_dim, 128) : 0;
+    if (estmm_pipe_wanted(r)) return estmm_plan_cap(r.T, r.k, r.E, tiles, cus);
+    return std::max(estmm_plan_cap(r.T, r.k, r.E), tiles ? estmm_plan_cap(r.T, r.k, r.E, tiles, 4 * cus) : 0);
+}
+
+int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, int cap, hipStream_t st) {
     if (r.E > 4096) HEXA_FAIL(HEXA_ERR_UNSUPPORTED, "estmm plan: more than 4096 experts");
-    hipLaunchKernelGGL(estmm_plan_kernel, dim3(1), dim3(256), 2 * r.E * sizeof(int), st, plan, r.offsets, r.E, r.k,
-                       estmm_plan_cap(r.T, r.k, r.E), max_slots);
+    hipLaunchKernelGGL(estmm_plan_kernel, dim3(1), dim3(256), 2 * r.E * sizeof(int), st, plan, r.offsets, r.E, r.k, cap,
+                       max_slots);
     HEXA_CHECK_LAUNCH("estmm_plan");
     return HEXA_OK;
 }

@@ -102,6 +102,7 @@ enum Opt {
     OPT_BATCH,          // HEXA_MOE_BATCH: 2 = every small kernel of the depth backward in a launch of its own, 1 = four batch launches instead of three
     OPT_FFN_FUSED,      // HEXA_MOE_FFN_FUSED: 1 = hexa_moe_depth_forward runs fc1, GELU and fc2 in one kernel where it is covered
     OPT_GATE_ROUTER,    // HEXA_MOE_GATE_ROUTER: 2 = hexa_moe_depth_forward runs the gate projection and the router as two launches
+    OPT_ESTMM_PIPE,     // HEXA_ESTMM_PIPE: 1 = the persistent ESTMM kernel wherever it applies (default: the one-item-per-workgroup kernel)
     OPT_COUNT
 };
 int option(int id);
@@ -115,7 +116,13 @@ int launch_ffn16_fused(void* y1, void* y2, void* y, const void* x, const void* w
                        const void* b2, const RouteView& r, int d_in, int hidden, int d_out, int act_dt, int b1_dt,
                        int b2_dt, void* slot_ws, hipStream_t st);
 int launch_colsum_fold(const EsmmArgs& a, int mt_ub, int tile_rows, int ntn, int bn, hipStream_t st);
-int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, hipStream_t st);
+int estmm_plan_cap_for(const RouteView& r, int out_dim, int in_dim);   // rows above which an expert's list is cut
+int launch_estmm_plan(int32_t* plan, const RouteView& r, int max_slots, int cap, hipStream_t st);
+int launch_estmm_fixup(const EstmmArgs& a, hipStream_t st);
+// whether a routing of this size goes to the persistent ESTMM kernel (the plan is made for the kernel that will run)
+bool estmm_pipe_wanted(const RouteView& r);
+bool estmm16_pipe_supported(const EstmmArgs& a);
+int launch_estmm16_pipe(const EstmmArgs& a, hipStream_t st);
 int launch_esmm16_dma(const EsmmArgs& a, hipStream_t s);
 bool dma_path_enabled();
 bool estmm16_dma_supported(const EstmmArgs& a);
@@ -137,7 +144,7 @@ int launch_gate_router(float* logits, float* scores, int32_t* idx, const void* x
                        float noise_scale, int T, int d, int E, int k, int x_dt, float* ws, int32_t* hist, hipStream_t st);
 int launch_route_from_hist(const int32_t* idx, int T, int k, int E, int32_t* route, int32_t* hist, int unit_tokens,
                            float* l_aux, float* me, float* ce, const float* router_ws, int32_t* plan, int plan_slots,
-                           hipStream_t st);
+                           int plan_cap, hipStream_t st);
 int launch_gelu_bwd(void* dy1, const void* dy2, const void* y1, int64_t n, int dt, hipStream_t s);
 
 // ---- small device helpers -------------------------------------------------------------------

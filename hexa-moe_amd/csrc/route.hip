@@ -704,7 +704,7 @@ namespace hexa {
 // router_ws) and scatter (+ the ESTMM work plan, when plan is given).
 int launch_route_from_hist(const int32_t* idx, int T, int k, int E, int32_t* route, int32_t* hist, int unit_tokens,
                            float* l_aux, float* me, float* ce, const float* router_ws, int32_t* plan, int plan_slots,
-                           hipStream_t st) {
+                           int plan_cap, hipStream_t st) {
     hexa_route_layout L;
     hexa_route_layout_get(T, k, E, &L);
     const int units = div_up(T, unit_tokens);
@@ -717,7 +717,7 @@ int launch_route_from_hist(const int32_t* idx, int T, int k, int E, int32_t* rou
                            hist, route + L.counts, route + L.offsets, reinterpret_cast<int4*>(route + L.tile_info),
                            route + L.tile_count, L.mt_ub, reinterpret_cast<int4*>(route + L.tile_info_l), route + L.tile_count_l,
                            L.mt_ub_l, route + L.token_ids, route + L.expert_ids, l_aux, me, ce, router_ws,
-                           router_ws ? router_ws + (size_t)units * E : nullptr, plan, estmm_plan_cap(T, k, E), plan_slots);
+                           router_ws ? router_ws + (size_t)units * E : nullptr, plan, plan_cap, plan_slots);
         HEXA_CHECK_LAUNCH("route_finish");
         return HEXA_OK;
     }
@@ -728,7 +728,7 @@ int launch_route_from_hist(const int32_t* idx, int T, int k, int E, int32_t* rou
     HEXA_CHECK_LAUNCH("route_scan_loss");
     hipLaunchKernelGGL(route_scatter_plan_kernel, dim3(units + (plan ? 1 : 0), k), dim3(kWave), sizeof(int32_t) * 2 * E, st, idx,
                        k, T, E, units, unit_tokens, ceil_log2(E), hist, route + L.offsets, route + L.token_ids,
-                       route + L.expert_ids, plan, estmm_plan_cap(T, k, E), plan_slots);
+                       route + L.expert_ids, plan, plan_cap, plan_slots);
     HEXA_CHECK_LAUNCH("route_scatter_plan");
     return HEXA_OK;
 }

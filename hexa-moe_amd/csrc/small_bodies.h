@@ -68,11 +68,18 @@ __device__ inline void router_loss_body(float* lds, float* __restrict__ l_aux, f
 // (bit-reproducible).  Units are numbered heaviest expert first.  plan = 4 arrays of E ints in rank
 // order -- expert, parts, first unit, first scratch slot -- followed by the number of units.
 // lds: 2 * E ints.
-constexpr int PLAN_MAX_PARTS = 4;
+constexpr int PLAN_MAX_PARTS = 8;
+constexpr int PLAN_QUEUE_INTS = 16;    // work counters of the persistent ESTMM kernel behind the plan (8 queues, a finish count)
+__host__ __device__ inline int estmm_plan_queue_at(int E) { return 4 * E + 1; }
 
-__host__ __device__ inline int estmm_plan_cap(long T, int k, int E) {   // parts for experts above 1.5x the mean load
+// An expert's list is cut when it is longer than `cap` rows.  The persistent kernel hands items (an expert's or
+// part's list x one 128 x 128 block of the result) longest-first to whichever workgroup is free, so a cut only pays
+// when one item would be longer than a workgroup's share of the launch: rows of all lists x blocks per expert /
+// workgroups (`tiles` = 0: unknown result size, the rule of the one-item-per-workgroup kernel: 1.5x the mean load).
+__host__ __device__ inline int estmm_plan_cap(long T, int k, int E, int tiles = 0, int workgroups = 256) {
     const long avg = T * k / E;
-    const long c = (3 * avg + 1) / 2;
+    long c = (3 * avg + 1) / 2;
+    if (tiles > 0) c = T * k * tiles / workgroups;
     return (int)(c > 256 ? c : 256);
 }
 
@@ -122,6 +129,7 @@ __device__ inline void estmm_plan_from_loads(int* sp, int* __restrict__ plan, in
         }
         plan[4 * E] = unit;
     }
+    if (threadIdx.x < PLAN_QUEUE_INTS) plan[estmm_plan_queue_at(E) + threadIdx.x] = 0;
 }
 
 // ---- ESS: per-expert column sums of gathered rows (see ess.hip) --------------------------------------------------
@@ -289,14 +297,19 @@ __device__ __forceinline__ void estmm_fixup_body(const FixupK& p, int block) {
     if (i >= p.mn) return;
     const int e = p.plan[r];
     const float* src = p.scratch + (size_t)p.plan[3 * E + r] * p.mn + i;
-    // every part's load in flight at once (at most PLAN_MAX_PARTS), added in part order
-    float4 w[PLAN_MAX_PARTS];
+    // four parts' loads in flight at once, added in part order
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int c0 = 0; c0 < n; c0 += 4) {
+        float4 w[4];
 #pragma unroll
-    for (int c = 0; c < PLAN_MAX_PARTS; ++c) w[c] = *reinterpret_cast<const float4*>(src + (size_t)min(c, n - 1) * p.mn);
-    float4 v = w[0];
+        for (int c = 0; c < 4; ++c) w[c] = *reinterpret_cast<const float4*>(src + (size_t)min(c0 + c, n - 1) * p.mn);
 #pragma unroll
-    for (int c = 1; c < PLAN_MAX_PARTS; ++c) {
-        if (c < n) { v.x += w[c].x; v.y += w[c].y; v.z += w[c].z; v.w += w[c].w; }
+        for (int c = 0; c < 4; ++c) {
+            if (c0 + c < n) {
+                if (c0 + c == 0) v = w[0];
+                else { v.x += w[c].x; v.y += w[c].y; v.z += w[c].z; v.w += w[c].w; }
+            }
+        }
     }
     const size_t o = (size_t)e * p.mn + i;
     if (!p.accumulate) {   // one store of the four results (mn is a multiple of 4, so the piece is aligned)

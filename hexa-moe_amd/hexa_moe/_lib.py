@@ -16,6 +16,11 @@ HEXA_TILE_ROWS = 128
 HEXA_TILE_ROWS_L = 256
 HEXA_ROUTE_UNIT = 512
 
+
+def estmm_plan_ints(num_experts):
+    """HEXA_ESTMM_PLAN_INTS of the header: ints of an ESTMM work plan (with the work queue's counters)."""
+    return 4 * int(num_experts) + 32
+
 _vp, _i, _i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
 
 
@@ -44,7 +49,7 @@ SIGNATURES = {
     "hexa_route_from_padded_lists": (_i, [_vp, _vp, _vp, _i64, _i, _i, _i, _vp, _vp]),
     "hexa_esmm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "hexa_estmm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp]),
-    "hexa_estmm_plan": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
+    "hexa_estmm_plan": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "hexa_ess": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
     "hexa_ess_noalloc": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "hexa_fused_grad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
@@ -86,7 +91,7 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.hexa_abi_version() != 8:
+    if lib.hexa_abi_version() != 9:
         raise RuntimeError("hexa_moe: libhexa_moe_hip.so has an unexpected ABI version")
     _lib = lib
     return lib

@@ -216,8 +216,8 @@ class FusedMoEDepth(torch.autograd.Function):
         state = torch.empty(2 * T * E + T + nstats, dtype=torch.float32, device=dev)
         logits, scores = state[:T * E], state[T * E:2 * T * E]
         thr, stats = state[2 * T * E:2 * T * E + T], state[2 * T * E + T:]
-        ints = torch.empty(T * top_k + 4 * E + 1, dtype=torch.int32, device=dev)
-        idx, estmm_plan = ints[:T * top_k].view(T, top_k), ints[T * top_k:]   # the backward's ESTMM work plan: 4E+1 ints
+        ints = torch.empty(T * top_k + _lib.estmm_plan_ints(E), dtype=torch.int32, device=dev)
+        idx, estmm_plan = ints[:T * top_k].view(T, top_k), ints[T * top_k:]   # the backward's ESTMM work plan
         noise = torch.randn(T, E, dtype=torch.float32, device=dev) if noise_scale > 0 else None
         blob = config.route_pool.slot(config.stage, T, top_k, E, dev)
         y12 = torch.empty(2, top_k, T, hidden, dtype=x.dtype, device=dev)

@@ -76,16 +76,18 @@ class Route:
         self.layout = _lib.route_layout(T, k, E)
         self._plans = {}
 
-    def estmm_plan(self, max_slots):
-        """Work plan of estmm for this routing (int32 [4E+1]); made on first use, then shared by every
-        estmm call on the routing."""
-        plan = self._plans.get(max_slots)
+    def estmm_plan(self, max_slots, out_dim=0, in_dim=0):
+        """Work plan of estmm for this routing and result size (int32 [HEXA_ESTMM_PLAN_INTS]); made on first use,
+        then shared by every estmm call on the routing whose result has as many 128 x 128 blocks.  The plan also
+        holds the work queue of the persistent kernel, so calls that use it must not overlap (one stream)."""
+        key = (int(max_slots), -(-int(out_dim) // 128) * -(-int(in_dim) // 128))
+        plan = self._plans.get(key)
         if plan is None:
-            plan = torch.empty(4 * self.E + 1, dtype=torch.int32, device=self.blob.device)
+            plan = torch.empty(_lib.estmm_plan_ints(self.E), dtype=torch.int32, device=self.blob.device)
             rc = _call("estmm_plan", _lib.load().hexa_estmm_plan, _ptr(plan), _ptr(self.blob), self.T, self.k, self.E,
-                       int(max_slots), _stream())
+                       int(max_slots), int(out_dim), int(in_dim), _stream())
             _lib.check(rc, "hexa_estmm_plan")
-            self._plans[max_slots] = plan
+            self._plans[key] = plan
         return plan
 
     def _part(self, start, n):
@@ -236,16 +238,18 @@ def estmm(dy, x, route, dy_per_slot, x_per_slot, out=None, out_dtype=torch.float
         out = torch.empty(E, out_dim, in_dim, dtype=out_dtype, device=x.device)
     plan = scratch = None
     slots = 0
-    if x.dtype != torch.float32 and T * k >= 128 * E:
-        # the busiest experts are cut into parts: a plan (made once per routing) and scratch for up to 2E fp32
-        # partial results, at most 256 MiB
-        slots = min(2 * E, (256 << 20) // (out_dim * in_dim * 4))
-        if slots >= 2 and (out_dim * in_dim) % 4 == 0:
-            plan = route.estmm_plan(slots)
+    if x.dtype != torch.float32:
+        # a plan (made once per routing and result size) orders the work of the persistent kernel; with lists long
+        # enough to be worth cutting it comes with scratch for up to 2E fp32 partial results, at most 256 MiB
+        if T * k >= 128 * E and (out_dim * in_dim) % 4 == 0:
+            slots = min(2 * E, (256 << 20) // (out_dim * in_dim * 4))
+            slots = slots if slots >= 2 else 0
+        plan = route.estmm_plan(slots, out_dim, in_dim)
+        if slots:
             scratch = torch.empty(slots * out_dim * in_dim, dtype=torch.float32, device=x.device)
     rc = _call(f"estmm[{out_dim}x{in_dim}]", _lib.load().hexa_estmm, _ptr(out), _ptr(dy), _ptr(x), _ptr(route.blob),
                int(bool(dy_per_slot)), int(bool(x_per_slot)), int(bool(accumulate)), T, k, out_dim, in_dim, E,
-               _dt(x), _dt(out), _ptr(plan), slots if plan is not None else 0, _ptr(scratch), _stream())
+               _dt(x), _dt(out), _ptr(plan), slots, _ptr(scratch), _stream())
     _lib.check(rc, "hexa_estmm")
     return out
 
@@ -447,7 +451,7 @@ def _event_array(events):
 
 def moe_depth_forward(plan, x, wg, noise, fc1_w, fc1_b, fc2_w, fc2_b, logits, scores, idx, thr, stats, route_blob,
                       estmm_plan, y1, y2, y, ws, events=None):
-    """estmm_plan: int32 [4E+1] that receives the work plan of the backward's ESTMM calls, or None."""
+    """estmm_plan: int32 [_lib.estmm_plan_ints(E)] that receives the work plan of the backward's ESTMM calls, or None."""
     import ctypes
     _dev(x, wg, noise, fc1_w, fc1_b, fc2_w, fc2_b, idx, route_blob, y1, y2, y, ws)
     ev, nev = _event_array(events)

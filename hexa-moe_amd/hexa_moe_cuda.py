@@ -153,13 +153,13 @@ def _fused(j_b, j_x, j_w, j_y, w, x, token_idx_list, expert_idx_list, num_expand
     plan = scratch = ess_ws = None
     slots = 0
     mn = int(num_out_dims) * int(num_in_dims)
-    if j_y.dtype != torch.float32 and T * k >= 128 * E and mn % 4 == 0:
-        slots = min(2 * E, (256 << 20) // (mn * 4))
-        if slots >= 2:
-            plan = route.estmm_plan(slots)
+    if j_y.dtype != torch.float32:
+        if T * k >= 128 * E and mn % 4 == 0:
+            slots = min(2 * E, (256 << 20) // (mn * 4))
+            slots = slots if slots >= 2 else 0
+        plan = route.estmm_plan(slots, int(num_out_dims), int(num_in_dims))
+        if slots:
             scratch = torch.empty(slots * mn, dtype=torch.float32, device=j_y.device)
-        else:
-            slots = 0
     if j_b is not None and T * k >= 256 * E:
         ess_ws = torch.empty(8 * E * int(num_out_dims), dtype=torch.float32, device=j_y.device)
     rc = _lib.load().hexa_fused_grad(

@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define HEXA_ABI_VERSION 8
+#define HEXA_ABI_VERSION 9
 
 /* element types */
 #define HEXA_F32 0
@@ -140,23 +140,30 @@ int hexa_esmm(void* out, const void* x, const void* w, const void* bias, const i
  * dy_per_slot / x_per_slot say whether the operand is [k,T,*] (1) or [T,*] shared by the slots (0).
  * dt is the element type of dy and x (F32, F16 or BF16); dw_dt is F32 or dt.  Experts without tokens
  * get exact zeros (or are left untouched when accumulating).
- * plan / max_slots / scratch (optional; used by the 16-bit kernels): with a plan from hexa_estmm_plan for
- * the same routing and max_slots, experts with more than 1.5x the mean number of tokens are cut into up
- * to 4 parts that run as separate workgroups; the fp32 partial results go through `scratch`
- * (max_slots * out_dim * in_dim floats) and are added in a fixed order, so results stay bit-reproducible.
- * Without it one workgroup walks an expert's whole token list and the kernel is as slow as the busiest
- * expert.
+ * plan / max_slots / scratch (optional; used by the 16-bit kernels).  With a plan from hexa_estmm_plan for the same
+ * routing, max_slots and result size, the persistent kernel runs (up to 256 experts and 8 slots): one workgroup per
+ * CU takes (expert, 128 x 128 block) items from a queue, longest first, so the load balances without cutting
+ * experts; only an expert whose list is longer than a workgroup's share of the whole launch is cut into up to 8
+ * parts, whose fp32 partial results go through `scratch` (max_slots * out_dim * in_dim floats; max_slots < 2 or
+ * scratch == NULL: nothing is cut) and are added in a fixed order, so results stay bit-reproducible.  The plan
+ * also holds the queue's counters, which the call updates and leaves at zero: calls that share a plan must not
+ * overlap (calls on one stream do not).  Without a plan one workgroup walks an expert's whole token list per
+ * block and the kernel is as slow as the busiest expert.
  * Replaces the ESTMM task of FUSED_GRAD (kernels/fused_ops_full.cu:248-371). */
 int hexa_estmm(void* dw, const void* dy, const void* x, const int32_t* route, int dy_per_slot, int x_per_slot,
                int accumulate, int num_tokens, int top_k, int out_dim, int in_dim, int num_experts, int dt,
-               int dw_dt, const int32_t* plan, int max_slots, float* scratch, void* stream);
+               int dw_dt, int32_t* plan, int max_slots, float* scratch, void* stream);
 
-/* Work plan of hexa_estmm for one routing: 4*num_experts+1 ints (experts by decreasing load, their parts,
- * first work unit and first scratch slot, number of units).  Depends on the routing and max_slots only, so one
- * plan serves every hexa_estmm call of a layer's backward.  No counterpart in the reference, whose ESTMM
- * task walks each expert's list in one thread block (kernels/fused_ops_full.cu:248-371). */
+/* Work plan of hexa_estmm for one routing: HEXA_ESTMM_PLAN_INTS(num_experts) ints (experts by decreasing load,
+ * their parts, first work unit and first scratch slot, number of units, then the work queue's counters, zeroed).
+ * out_dim / in_dim: the size of the result the plan is for (0, 0: unknown -- experts above 1.5x the mean load are
+ * cut, the rule of the one-item-per-workgroup kernel).  Depends on the routing, max_slots and that size only, so
+ * one plan serves every hexa_estmm call of a layer's backward whose results have the same number of 128 x 128
+ * blocks.  No counterpart in the reference, whose ESTMM task walks each expert's list in one thread block
+ * (kernels/fused_ops_full.cu:248-371). */
+#define HEXA_ESTMM_PLAN_INTS(num_experts) (4 * (num_experts) + 32)
 int hexa_estmm_plan(int32_t* plan, const int32_t* route, int num_tokens, int top_k, int num_experts, int max_slots,
-                    void* stream);
+                    int out_dim, int in_dim, void* stream);
 
 /* ESS: db[e][o] (+)= sum over slots and tokens routed to e of dy[(s),t,o].
  * ws (optional, ws_floats floats of scratch; 8*num_experts*out_dim is enough): long token lists are then
@@ -196,7 +203,7 @@ int hexa_ess_noalloc(void* db, const void* dy, const int32_t* route, int dy_per_
 int hexa_fused_grad(void* j_b, void* j_x, void* j_w, const void* j_y, const void* w, const void* x,
                     const int32_t* route, int m2s, int accumulate, int num_tokens, int top_k, int in_dim,
                     int out_dim, int num_experts, int act_dt, int w_dt, int jx_dt, int jw_dt, int jb_dt,
-                    void* slot_ws, const int32_t* plan, int max_slots, float* estmm_scratch, float* ess_ws,
+                    void* slot_ws, int32_t* plan, int max_slots, float* estmm_scratch, float* ess_ws,
                     int64_t ess_ws_floats, void* stream);
 
 /* Steps 6-8 of the backward in one call: out[s][t][:] = (x[t][:] . w[e_s(t)]) * gelu'(y1[s][t][:]) (out, y1
@@ -295,9 +302,9 @@ int hexa_moe_depth_ws_bytes(const hexa_moe_depth_desc* d, int64_t* forward_bytes
  * stats / noise are ignored.
  * Then: route = hexa_route_build(idx); y1 = x.W1^T + b1 and y2 = gelu(y1) ([k][T][hidden], saved for the backward);
  * y [T][d_out] = sum over slots of y2.W2 + b2.  Biases may be NULL.
- * plan (may be NULL): 4*num_experts+1 ints that receive the work plan of the backward's ESTMM calls (as
- * hexa_estmm_plan; it depends on the routing only); hand the same buffer to hexa_moe_depth_backward and that call
- * skips making it.  (With the GShard loss and up to 240 experts the router, the loss, the routing pass and the plan
+ * plan (may be NULL): HEXA_ESTMM_PLAN_INTS(num_experts) ints that receive the work plan of the backward's ESTMM
+ * calls (as hexa_estmm_plan; it depends on the routing only); hand the same buffer to hexa_moe_depth_backward and
+ * that call skips making it.  (With the GShard loss and up to 240 experts the router, the loss, the routing pass and the plan
  * take two launches in all: the router counts its own tokens for the routing pass, whose one launch scatters the
  * tokens, finishes the loss and makes the plan.)
  * events (may be NULL): 2*n caller-owned hipEvent_t handles; pair i is recorded on `stream` around major kernel i
@@ -313,13 +320,14 @@ int hexa_moe_depth_forward(const hexa_moe_depth_desc* d, const void* x, const fl
  * loss carries no gradient).  Results (each may be NULL to skip it): dx [T][d_in] = the expert path's input
  * gradient plus, with wg, the gate path's; dwg [E][d_in] fp32; dw1 [E][hidden][d_in], db1 [E][hidden],
  * dw2 [E][hidden][d_out], db2 [E][d_out].  dy1 is caller memory for the hidden gradient ([k][T][hidden] of act_dt);
- * its contents after the call are dy1 = (dy.W2^T) * gelu'(y1).  plan: the buffer the forward filled, or NULL.
+ * its contents after the call are dy1 = (dy.W2^T) * gelu'(y1).  plan: the buffer the forward filled (its queue
+ * counters are used and left at zero), or NULL.
  * events: pairs around (0) the dy1 kernel with its bias-gradient sums, (1) the dx kernel and its slot sum,
  * (2) ESTMM dW2, (3) ESTMM dW1. */
 int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void* dy, const float* grad_l_aux, const void* x,
                             const float* wg, const void* fc1_w, const void* fc2_w, const float* scores,
                             const int32_t* idx, const float* thr, const float* stats, const int32_t* route,
-                            const int32_t* plan, const void* y1, const void* y2, void* dx, float* dwg, void* dw1,
+                            int32_t* plan, const void* y1, const void* y2, void* dx, float* dwg, void* dw1,
                             void* db1, void* dw2, void* db2, void* dy1, void* ws, int64_t ws_bytes, void* const* events,
                             int num_events, void* stream);
 

@@ -11,9 +11,9 @@ pytestmark = pytest.mark.gpu
 
 SETTINGS = [{"tile": t} for t in range(1, 12)] + [
     {"pipe": 1}, {"pipe": 2}, {"tile": 12}, {"tile": 13},
-    {"esmm_map": 2}, {"esmm_map": 2, "esmm_group": 16}, {"estmm_group": 1}, {"estmm_group": 4}, {"estmm_group": 12}, {"esmm_stream": 1}, {"esmm_stream": 2}, {"general_kernels": 1},
+    {"esmm_map": 2}, {"esmm_map": 2, "esmm_group": 16}, {"estmm_group": 1}, {"estmm_group": 4}, {"estmm_group": 12}, {"esmm_stream": 1}, {"esmm_stream": 2}, {"general_kernels": 1}, {"estmm_pipe": 1},
 ]
-ALL = ("tile", "pipe", "esmm_map", "esmm_group", "estmm_group", "esmm_stream", "general_kernels")
+ALL = ("tile", "pipe", "esmm_map", "esmm_group", "estmm_group", "esmm_stream", "general_kernels", "estmm_pipe")
 
 
 @pytest.fixture

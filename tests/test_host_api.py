@@ -33,7 +33,7 @@ def test_header_symbols_are_exported():
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in include/hexa_moe_hip.h but not exported"
     assert declared == set(_lib.SIGNATURES), "ctypes table and header disagree"
-    assert lib.hexa_abi_version() == 8
+    assert lib.hexa_abi_version() == 9
 
 
 def test_abi_argument_errors_without_a_gpu():

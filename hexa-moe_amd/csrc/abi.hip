@@ -28,6 +28,7 @@ OptEntry g_opts[OPT_COUNT] = {
     {"ffn_fused", "HEXA_MOE_FFN_FUSED", 0, false},
     {"gate_router", "HEXA_MOE_GATE_ROUTER", 0, false},
     {"estmm_pipe", "HEXA_ESTMM_PIPE", 0, false},
+    {"side_stream", "HEXA_MOE_SIDE_STREAM", 0, false},
 };
 }  // namespace
 

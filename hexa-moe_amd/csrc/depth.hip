@@ -6,6 +6,7 @@
 // Replaces the MoE branch of MoE_Cascaded.forward (hexa_moe_cuda/hexa_moe/impls/cascaded_moe.py:508-568),
 // FusedMoE_Shared_CudaCore.forward (impls/layers.py:99-277) and .backward (impls/layers.py:280-474).
 #include <algorithm>
+#include <mutex>
 
 #include "small_tasks.h"
 
@@ -27,19 +28,40 @@ struct Carver {   // hands out aligned pieces of the workspace; with base == nul
     }
 };
 
-// ESTMM scratch slots for the busiest experts' partial results (the same rule as the Python wrapper of the
-// single operator: up to 2E slots, at most 256 MiB, only for 16-bit operands with long enough lists)
+// ESTMM scratch slots for the partial results of experts whose lists are cut (up to E slots, at most 128 MiB per
+// result, only for 16-bit operands with long enough lists)
 int estmm_slots(const hexa_moe_depth_desc& d, int out_dim, int in_dim) {
     if (d.act_dt == HEXA_F32 || (int64_t)d.num_tokens * d.top_k < (int64_t)128 * d.num_experts) return 0;
     const int64_t mn = (int64_t)out_dim * in_dim;
     if (mn % 4) return 0;
-    const int64_t slots = std::min<int64_t>(2 * d.num_experts, ((int64_t)256 << 20) / (mn * 4));
+    const int64_t slots = std::min<int64_t>(d.num_experts, ((int64_t)128 << 20) / (mn * 4));
     return slots >= 2 ? (int)slots : 0;
+}
+
+// A second stream and the events that tie it to the caller's, made once per device (default priority; the first call
+// on a device must not be under stream capture).  The small kernels of the backward are bound by their latency
+// chains, not by the chip: beside the matmul kernels they cost next to nothing.
+struct SideStream { hipStream_t st = nullptr; hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr}; bool ok = false, tried = false; };
+SideStream* side_stream() {
+    static SideStream per_device[64];
+    static std::mutex mu;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    SideStream& s = per_device[dev];
+    if (!s.tried) {
+        s.tried = true;
+        bool ok = hipStreamCreateWithFlags(&s.st, hipStreamNonBlocking) == hipSuccess;
+        for (int i = 0; ok && i < 4; ++i) ok = hipEventCreateWithFlags(&s.ev[i], hipEventDisableTiming) == hipSuccess;
+        if (!ok) (void)hipGetLastError();
+        s.ok = ok;
+    }
+    return s.ok ? &s : nullptr;
 }
 
 struct FwdWs { float* router; int32_t* hist; void* slot_ws; int64_t bytes; };
 struct BwdWs {
-    float* dlogits; float* gate; float* ess; float* colsum; int64_t colsum_floats; int32_t* plan; float* estmm;
+    float* dlogits; float* gate; float* ess; float* colsum; int64_t colsum_floats; int32_t* plan; float* estmm; float* estmm2;
     int slots; void* slot_ws; void* dx_gate; int64_t bytes;
 };
 
@@ -67,13 +89,13 @@ int carve_backward(const hexa_moe_depth_desc& d, void* ws, BwdWs* out) {
     out->ess = static_cast<float*>(c.take((int64_t)8 * E * d.d_out * 4));
     out->colsum = static_cast<float*>(c.take(cf * 4));
     out->colsum_floats = cf;
-    // one plan and one scratch area serve both ESTMM calls (they run one after the other on the stream)
+    // one plan serves both ESTMM calls; each has a scratch area of its own (the fix-up of the first may run on the
+    // side stream while the second call's kernel writes its partial results)
     const int s2 = estmm_slots(d, d.hidden, d.d_out), s1 = estmm_slots(d, d.hidden, d.d_in);
     out->slots = std::min(s1, s2);
     out->plan = static_cast<int32_t*>(c.take((int64_t)HEXA_ESTMM_PLAN_INTS(E) * 4));
-    out->estmm = out->slots >= 2
-                     ? static_cast<float*>(c.take((int64_t)out->slots * d.hidden * std::max(d.d_in, d.d_out) * 4))
-                     : nullptr;
+    out->estmm = out->slots >= 2 ? static_cast<float*>(c.take((int64_t)out->slots * d.hidden * d.d_out * 4)) : nullptr;
+    out->estmm2 = out->slots >= 2 ? static_cast<float*>(c.take((int64_t)out->slots * d.hidden * d.d_in * 4)) : nullptr;
     out->slot_ws = k > 1 ? c.take((int64_t)(k - 1) * T * d.d_in * elem_size(d.act_dt)) : nullptr;
     out->dx_gate = c.take((int64_t)T * d.d_in * elem_size(d.act_dt));
     out->bytes = c.used;
@@ -239,6 +261,19 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
     struct Guard { ~Guard() { defer_targets() = DeferTargets(); } } guard;
     DeferTargets& tg = defer_targets();
     hipStream_t st = (hipStream_t)stream;
+    // With the side stream the batches B and C and the gate's backward run beside the matmul kernels:
+    //   caller's stream:  ESTMM dW2 | dy1 kernel | ESTMM dW1 |            dx kernel | D
+    //   side stream:                 B | gate backward        | C
+    // B waits for ESTMM dW2 (event 0), the dx kernel for the gate's backward (event 1), C for ESTMM dW1 (event 2), the
+    // caller's stream for C (event 3) before the call's last launch.
+    SideStream* side = batching && !early_a && option(OPT_SIDE_STREAM) == 1 ? side_stream() : nullptr;
+    hipStream_t sst = side ? side->st : st;
+    auto hand_over = [&](int i, hipStream_t from, hipStream_t to) -> int {   // `to` continues behind what `from` holds now
+        if (!side) return HEXA_OK;
+        if (hipEventRecord(side->ev[i], from) != hipSuccess || hipStreamWaitEvent(to, side->ev[i], 0) != hipSuccess)
+            HEXA_FAIL(HEXA_ERR_LAUNCH, "hexa_moe_depth_backward: event hand-over between the streams failed");
+        return HEXA_OK;
+    };
 
     // step 4: db2 = ESS(dy)
     if (db2) {
@@ -271,7 +306,8 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
         RUN(ev.end(2));
         tg = DeferTargets();
     }
-    RUN(batch_flush(B, st));
+    RUN(hand_over(0, st, sst));
+    RUN(batch_flush(B, sst));
     if (dx || dw1 || db1) {
         // steps 6-8: dy1 = (dy . W2^T) * gelu'(y1), db1 = ESS(dy1)
         if (batching) tg.colsum_fold = &C;
@@ -289,7 +325,7 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
             if (batching) tg.fixup = &C;
             RUN(ev.begin(3));
             RUN(hexa_estmm(dw1, dy1, x, route, 1, 0, 0, T, k, d->hidden, d->d_in, E, d->act_dt, d->gw1_dt,
-                           planned ? w.plan : nullptr, planned ? w.slots : 0, planned && w.slots >= 2 ? w.estmm : nullptr, stream));
+                           planned ? w.plan : nullptr, planned ? w.slots : 0, planned && w.slots >= 2 ? w.estmm2 : nullptr, stream));
             RUN(ev.end(3));
             tg = DeferTargets();
         }
@@ -305,10 +341,12 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
                                                         d->act_dt, w.slot_ws);
         if (batching) tg.dwg_reduce = &D;
         RUN(hexa_gate_backward(dx ? (gate_dx_in_ws ? w.dx_gate : dx) : nullptr, dwg, w.dlogits, x, wg, T, d->d_in, E,
-                               d->act_dt, w.gate, stream));
+                               d->act_dt, w.gate, sst));
         tg = DeferTargets();
     }
-    RUN(batch_flush(C, st));
+    RUN(hand_over(1, sst, st));
+    RUN(hand_over(2, st, sst));
+    RUN(batch_flush(C, sst));
     // step 10: dx = ESMM(dy1, W1), summed over the slots (+ the gate's share)
     if (dx) {
         if (batching) tg.sum_slots = &D;
@@ -323,5 +361,6 @@ extern "C" int hexa_moe_depth_backward(const hexa_moe_depth_desc* d, const void*
         tg = DeferTargets();
     }
     RUN(batch_flush(D, st));
+    RUN(hand_over(3, sst, st));
     return HEXA_OK;
 }

@@ -103,6 +103,7 @@ enum Opt {
     OPT_FFN_FUSED,      // HEXA_MOE_FFN_FUSED: 1 = hexa_moe_depth_forward runs fc1, GELU and fc2 in one kernel where it is covered
     OPT_GATE_ROUTER,    // HEXA_MOE_GATE_ROUTER: 2 = hexa_moe_depth_forward runs the gate projection and the router as two launches
     OPT_ESTMM_PIPE,     // HEXA_ESTMM_PIPE: 1 = the persistent ESTMM kernel wherever it applies (default: the one-item-per-workgroup kernel)
+    OPT_SIDE_STREAM,    // HEXA_MOE_SIDE_STREAM: the small kernels of hexa_moe_depth_backward on a second stream beside the matmul kernels: 1 = yes, 2 = no
     OPT_COUNT
 };
 int option(int id);

@@ -239,15 +239,19 @@ def test_nan_token_row_stays_routed_and_propagates(dev, loss):
 @pytest.mark.parametrize("loss", ["gshard", "load_importance"])
 @pytest.mark.parametrize("dtype,k,bias", [(torch.float32, 1, True), (torch.bfloat16, 2, True), (torch.float16, 2, False),
                                           (torch.bfloat16, 1, True)])
-@pytest.mark.parametrize("batch", [0, 1, 2])
+@pytest.mark.parametrize("batch", [0, 1, 2, "side"])
 def test_depth_call_equals_operator_by_operator(dev, dtype, k, bias, loss, batch):
     """hexa_moe_depth_forward / _backward (one library call per direction) run the same kernels in the same
     order as the per-operator path: same routing, identical y, l_aux and parameter gradients; dx differs only
     by where the gate path's share is added (inside the slot sum instead of a separate addition)."""
     from hexa_moe import _lib
     E, d, T = 16, 256, 2500
-    # batch 2: every small kernel of the backward in a launch of its own instead of the three batch launches; 1: four
+    # batch 2: every small kernel of the backward in a launch of its own instead of the three batch launches; 1: four;
+    # "side": the batches and the gate's backward on the library's second stream, beside the matmul kernels
+    side = batch == "side"
+    batch = 0 if side else batch
     _lib.check(_lib.load().hexa_set_option(b"batch", batch), "hexa_set_option")
+    _lib.check(_lib.load().hexa_set_option(b"side_stream", 1 if side else 2), "hexa_set_option")
     m = _module([d], [0], E=E, k=k, bias=bias, act=F.gelu, noise=1.0).to(dev).to(dtype).eval()
     m.gates[0].wg.weight.data = m.gates[0].wg.weight.data.float()
     m.is_gshard_loss = loss == "gshard"
@@ -268,6 +272,7 @@ def test_depth_call_equals_operator_by_operator(dev, dtype, k, bias, loss, batch
             grads += [m.batched_fc1_bias[0].grad.clone(), m.batched_fc2_bias[0].grad.clone()]
         res.append((m.dispatch_params.routing_.clone().long(), y.detach().clone(), l_aux.detach().clone(), xi.grad.clone(), grads))
     _lib.check(_lib.load().hexa_set_option(b"batch", 0), "hexa_set_option")
+    _lib.check(_lib.load().hexa_set_option(b"side_stream", 0), "hexa_set_option")
     (ra, ya, la, dxa, ga), (rb, yb, lb, dxb, gb) = res
     assert torch.equal(ra, rb) and torch.equal(ya, yb) and torch.equal(la, lb)
     for u, v in zip(ga, gb):

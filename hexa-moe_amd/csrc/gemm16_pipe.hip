@@ -2,14 +2,14 @@
 // tiles, and the three phases a one-tile-per-workgroup kernel runs one after the other -- gathering operands,
 // MFMA main loop, activation + store epilogue -- run side by side on different wavefronts:
 //
-//   * 8 "multiply" wavefronts (4 x 2, 64 x 64 results each): LDS fragment reads and v_mfma_f32_32x32x16, nothing
-//     else.  They never touch global memory, so they never wait for it.
+//   * 4 "multiply" wavefronts (2 x 2, 64 x 64 results each, one per SIMD): LDS fragment reads and
+//     v_mfma_f32_32x32x16, nothing else.  They never touch global memory, so they never wait for it.
 //   * 4 "copy" wavefronts issue every asynchronous global->LDS copy (three stages deep, the pipeline never drains
 //     between tiles: the first stages of the next tile are issued during the last steps of the current one; the
 //     next tile's token ids and bias arrive by copy a whole tile ahead; the tile records of the workgroup's whole
 //     walk sit in LDS from the start).  They issue no stores, so their vmcnt counter only ever sees copies and the
 //     waits for a stage are exact.
-//   * 4 "store" wavefronts take the previous tile's rounded result out of an LDS staging area, apply the
+//   * 8 "store" wavefronts take the previous tile's rounded result out of an LDS staging area, apply the
 //     activation (GELU with a second output, or the GELU' factor read from the forward's pre-activation), and
 //     store 16-byte row pieces, spread over the main-loop steps of the tile that is being multiplied.
 //
@@ -53,8 +53,7 @@ using CfgP = Cfg<PIPE_WR, 2, PIPE_RB, 2, 3, 3, 64>;   // 128 x 128: 4 multiply w
 // any bit), as bf16 for GELU and as fp32 for GELU' (which is multiplied before rounding).  Entry 2 * (magnitude bits
 // - LUT_M_LO) + sign: the two 16-bit values of a 32-bit word are turned into two table addresses with packed 16-bit
 // arithmetic (four vector instructions per element instead of nine).  A piece with a value outside that range
-// (zeros, |x| >= 8, NaN) takes the polynomial: one wavefront-wide branch per 16-byte piece.  The fused epilogues are
-// bound by their vector instructions.
+// (zeros, |x| >= 8, NaN) takes the polynomial: one wavefront-wide branch per 16-byte piece.
 constexpr unsigned LUT_M_HI = 0x4100;
 template <typename TC, int ACT, bool COLSUM> constexpr unsigned pipe_lut_lo() {
     // GELU' with column sums: fp32 entries next to the column-sum area leave room for magnitudes from 2^-14 only

@@ -733,8 +733,8 @@ int launch_estmm_fixup(const EstmmArgs& a, hipStream_t st) {
     const long mn = (long)a.m_dim * a.n_dim;
     SmallTask t;
     t.kind = TASK_FIXUP;
-    t.fixup = FixupK{a.dw, a.plan, a.scratch, a.r.E, mn, a.dw_dt, a.accumulate, (int)((mn / 4 + 255) / 256)};
-    t.blocks = t.fixup.gx * a.r.E;
+    t.fixup = FixupK{a.dw, a.plan, a.scratch, a.r.E, mn, a.dw_dt, a.accumulate, (int)((mn / 4 + 256 * FIXUP_PIECES - 1) / (256 * FIXUP_PIECES))};
+    t.blocks = t.fixup.gx * std::min(a.r.E, std::max(1, a.max_slots / 2));   // (result piece, j-th cut expert)
     if (!defer_task(defer_targets().fixup, t)) {
         hipLaunchKernelGGL(estmm_fixup_kernel, dim3(t.blocks), dim3(256), 0, st, t.fixup);
         HEXA_CHECK_LAUNCH("estmm_fixup");

@@ -288,48 +288,67 @@ __device__ __forceinline__ void router_bwd_body(float* s_c, const RouterBwdK& p,
 }
 
 // dw[e] (+)= slot[0] + slot[1] + ... for the experts that the ESTMM plan cut into parts
+constexpr int FIXUP_PIECES = 4;   // pieces of 1024 results per fix-up workgroup
 __device__ __forceinline__ void estmm_fixup_body(const FixupK& p, int block) {
-    const int bx = block % p.gx, r = block / p.gx;
-    const int E = p.E;
+    // Workgroups (bx, j): piece bx of the result of the j-th expert whose list was cut.  A cut expert holds at least
+    // two scratch slots, so the launch has max_slots / 2 values of j and not one per expert -- with 32 experts of
+    // 3072 x 768 results and no list cut, one per expert was 74 thousand workgroups that only looked and left, 35 us.
+    const int bx = block % p.gx, j = block / p.gx;
+    const int E = p.E, lane = threadIdx.x & 63;
+    int r = -1;
+    for (int r0 = 0, seen = 0; r0 < E && r < 0; r0 += 64) {
+        const bool cut = r0 + lane < E && p.plan[E + r0 + lane] > 1;
+        unsigned long long m = __builtin_amdgcn_ballot_w64(cut);
+        const int c = __builtin_popcountll(m);
+        if (j < seen + c) {
+            for (int q = j - seen; q > 0; --q) m &= m - 1;
+            r = r0 + (int)__builtin_ctzll(m);
+        }
+        seen += c;
+    }
+    if (r < 0) return;
     const int n = p.plan[E + r];
-    if (n <= 1) return;
-    const long i = ((long)bx * 256 + threadIdx.x) * 4;
-    if (i >= p.mn) return;
     const int e = p.plan[r];
-    const float* src = p.scratch + (size_t)p.plan[3 * E + r] * p.mn + i;
-    // four parts' loads in flight at once, added in part order
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int c0 = 0; c0 < n; c0 += 4) {
-        float4 w[4];
+    const float* src0 = p.scratch + (size_t)p.plan[3 * E + r] * p.mn;
+    // FIXUP_PIECES pieces of 1024 results per workgroup, one after the other
+    for (int it = 0; it < FIXUP_PIECES; ++it) {
+        const long i = (((long)bx * FIXUP_PIECES + it) * 256 + threadIdx.x) * 4;
+        if (i >= p.mn) return;
+        const float* src = src0 + i;
+        // four parts' loads in flight at once, added in part order
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int c0 = 0; c0 < n; c0 += 4) {
+            float4 w[4];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) w[c] = *reinterpret_cast<const float4*>(src + (size_t)min(c0 + c, n - 1) * p.mn);
+            for (int c = 0; c < 4; ++c) w[c] = *reinterpret_cast<const float4*>(src + (size_t)min(c0 + c, n - 1) * p.mn);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            if (c0 + c < n) {
-                if (c0 + c == 0) v = w[0];
-                else { v.x += w[c].x; v.y += w[c].y; v.z += w[c].z; v.w += w[c].w; }
+            for (int c = 0; c < 4; ++c) {
+                if (c0 + c < n) {
+                    if (c0 + c == 0) v = w[0];
+                    else { v.x += w[c].x; v.y += w[c].y; v.z += w[c].z; v.w += w[c].w; }
+                }
             }
         }
-    }
-    const size_t o = (size_t)e * p.mn + i;
-    if (!p.accumulate) {   // one store of the four results (mn is a multiple of 4, so the piece is aligned)
-        typedef __attribute__((ext_vector_type(4))) float f4;
-        typedef __attribute__((ext_vector_type(2))) unsigned u2;
-        if (p.dw_dt == HEXA_F32) {
-            f4 w4 = {v.x, v.y, v.z, v.w};
-            *reinterpret_cast<f4*>(reinterpret_cast<float*>(p.dw) + o) = w4;
-        } else {
-            union { __bf16 b[4]; _Float16 h[4]; u2 w; } pk;   // the conversions of store_out
-            if (p.dw_dt == HEXA_BF16) { pk.b[0] = (__bf16)v.x; pk.b[1] = (__bf16)v.y; pk.b[2] = (__bf16)v.z; pk.b[3] = (__bf16)v.w; }
-            else { pk.h[0] = (_Float16)v.x; pk.h[1] = (_Float16)v.y; pk.h[2] = (_Float16)v.z; pk.h[3] = (_Float16)v.w; }
-            *reinterpret_cast<u2*>(reinterpret_cast<unsigned short*>(p.dw) + o) = pk.w;
+        const size_t o = (size_t)e * p.mn + i;
+        if (!p.accumulate) {   // one store of the four results (mn is a multiple of 4, so the piece is aligned)
+            typedef __attribute__((ext_vector_type(4))) float f4;
+            typedef __attribute__((ext_vector_type(2))) unsigned u2;
+            if (p.dw_dt == HEXA_F32) {
+                f4 w4 = {v.x, v.y, v.z, v.w};
+                *reinterpret_cast<f4*>(reinterpret_cast<float*>(p.dw) + o) = w4;
+            } else {
+                union { __bf16 b[4]; _Float16 h[4]; u2 w; } pk;   // the conversions of store_out
+                if (p.dw_dt == HEXA_BF16) { pk.b[0] = (__bf16)v.x; pk.b[1] = (__bf16)v.y; pk.b[2] = (__bf16)v.z; pk.b[3] = (__bf16)v.w; }
+                else { pk.h[0] = (_Float16)v.x; pk.h[1] = (_Float16)v.y; pk.h[2] = (_Float16)v.z; pk.h[3] = (_Float16)v.w; }
+                *reinterpret_cast<u2*>(reinterpret_cast<unsigned short*>(p.dw) + o) = pk.w;
+            }
+            continue;
         }
-        return;
+        store_out(p.dw, o, v.x, p.dw_dt, true);
+        store_out(p.dw, o + 1, v.y, p.dw_dt, true);
+        store_out(p.dw, o + 2, v.z, p.dw_dt, true);
+        store_out(p.dw, o + 3, v.w, p.dw_dt, true);
     }
-    store_out(p.dw, o, v.x, p.dw_dt, true);
-    store_out(p.dw, o + 1, v.y, p.dw_dt, true);
-    store_out(p.dw, o + 2, v.z, p.dw_dt, true);
-    store_out(p.dw, o + 3, v.w, p.dw_dt, true);
 }
 
 // db[e][n] (+)= the column sums an ESMM launch left per (slot, row tile, column tile), added in tile order.

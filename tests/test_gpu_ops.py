@@ -162,6 +162,32 @@ def test_estmm_16bit_result(dev, dtype):
     assert_close(db, O.ess(dy.float(), token_ids, offsets, True, E), TOL[dtype], "ess 16-bit result")
 
 
+def test_estmm_many_cut_experts(dev):
+    """More than 64 experts whose lists the plan cuts (70 of 1000 experts hold every token): the fix-up task finds
+    the j-th cut expert of the plan beyond the first 64 ranks, and workgroups past the last cut expert do nothing."""
+    from hexa_moe import ops
+    E, busy, rows, M, N = 1000, 70, 1900, 64, 64
+    T = busy * rows
+    g = gen(311)
+    experts = torch.randperm(E, generator=g)[:busy]
+    routing = experts[torch.randint(0, busy, (T, 1), generator=g)]
+    _, offsets, token_ids = O.route_build(routing, E)
+    dy = torch.randn(1, T, M, generator=g).to(BF16)
+    x = torch.randn(T, N, generator=g).to(BF16)
+    want = O.estmm(dy.float(), x.float(), token_ids, offsets, True, E)
+    route = ops.route_build(routing.to(dev), E)
+    got = ops.estmm(dy.to(dev), x.to(dev), route, True, False)
+    plan = next(iter(route._plans.values())).cpu()
+    assert int((plan[E:2 * E] > 1).sum()) == busy, "every busy expert's list is cut"
+    again = ops.estmm(dy.to(dev), x.to(dev), route, True, False)
+    torch.cuda.synchronize()
+    assert_close(got, want, 1e-4, "estmm with 70 cut experts")
+    assert torch.equal(got, again)
+    idle = torch.ones(E, dtype=torch.bool)
+    idle[experts] = False
+    assert float(got[idle.to(dev)].abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("per_slot", [False, True])
 def test_ess_long_lists(dev, dtype, per_slot):

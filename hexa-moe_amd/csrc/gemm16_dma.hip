@@ -817,9 +817,22 @@ int launch_estmm16_dma(const EstmmArgs& a, hipStream_t st) {
 // the 128x384 tile, whose rows have 48 pieces); the pipelined kernel has its own.
 // The pipelined persistent kernel runs whatever it covers (option "pipe": 2 = never, 1 = also when a tile shape is
 // forced); the one-tile kernels run the rest.
+// One exception by default: a plain launch (no fused activation) whose tiles come to between one and two per CU.  The
+// persistent kernel gives every CU a whole number of tiles, so half the CUs would idle through the second half of
+// the launch, while two one-tile workgroups share a CU at little loss (measured at 4608 rows, 3072 -> 768, 32
+// experts: 62 against 67 us; below one tile per CU -- 2304 rows -- the persistent kernel wins, 39 against 52 us).
+// The tile count is bounded from the host's side only (one partial tile per routing segment).
 static bool use_pipe(const EsmmArgs& a) {
     const int o = option(OPT_PIPE);
-    return o != 2 && (o == 1 || forced_tile() == 0) && esmm16_pipe_supported(a);
+    if (o == 2 || !(o == 1 || forced_tile() == 0) || !esmm16_pipe_supported(a)) return false;
+    if (o == 0 && a.act == HEXA_ACT_NONE && !a.colsum) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8)
+            cus = 256;
+        const long tiles_ub = (long)a.r.k * a.r.mt_ub * div_up(a.out_dim, 128);
+        if (4 * tiles_ub > 5 * (long)cus && tiles_ub <= 2 * (long)cus) return false;
+    }
+    return true;
 }
 
 bool esmm16_dma_colsum_supported(const EsmmArgs& a) {

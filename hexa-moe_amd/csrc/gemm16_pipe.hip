@@ -24,9 +24,9 @@
 // LDS accesses outside the MFMA fragment reads are inline assembly: a compiler-visible LDS access next to
 // copies in flight may be ordered behind them with s_waitcnt vmcnt(0), which would drain the pipeline.
 //
-// Covers: 16-bit operands and result, weights of the operands' type, in_dim a multiple of 32 and >= 128,
-// out_dim a multiple of 8, per-slot results (with or without activation / column sums) and slot-summed
-// results through scratch.  Everything else stays on esmm16_dma_kernel.
+// Covers: 16-bit operands and result, weights of the operands' type, in_dim a multiple of 64 and >= 256,
+// out_dim a multiple of 8, per-slot results (with or without activation / column sums; plain ones also
+// accumulating) and slot-summed results through scratch.  Everything else stays on esmm16_dma_kernel.
 //
 // Replaces esmm_shared_tensor_kernel_vectorized_accum_half (kernels/esmm_half.cu) and the ESMM task of the
 // fused backward kernels (kernels/fused_ops_half.cu) for the cases above.
@@ -452,6 +452,13 @@ __global__ __launch_bounds__(C::NT + 64 * (PIPE_COPY_WAVES + PIPE_STORE_WAVES)) 
         const unsigned boff = row_offset(t, tok);
         char* const outb = reinterpret_cast<char*>(t.to_ws ? p.ws : p.out);
         unsigned vw[4] = {val.x, val.y, val.z, val.w};
+        if (ACT == HEXA_ACT_NONE && p.accumulate) {   // result += : the rounded product joins what the row piece holds
+            const u32x4 old = *reinterpret_cast<const u32x4*>(outb + boff);
+            const unsigned ow[4] = {old.x, old.y, old.z, old.w};
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                vw[u] = pack2<TC>(lo16<TC>(vw[u]) + lo16<TC>(ow[u]), hi16<TC>(vw[u]) + hi16<TC>(ow[u]));
+        }
         if (ACT == HEXA_ACT_GELU_BWD) {
             const unsigned yw[4] = {y1v.x, y1v.y, y1v.z, y1v.w};
             bool looked_up = false;
@@ -635,7 +642,9 @@ bool esmm16_pipe_supported(const EsmmArgs& a) {
     using C = CfgP;
     if (!(a.w_dt == a.x_dt && a.out_dt == a.x_dt && (a.in_dim % C::BKC) == 0 && a.in_dim >= (2 * C::STAGES - 2) * C::BKC && (a.out_dim % 8) == 0))
         return false;
-    if (a.accumulate || a.r.k > 8) return false;
+    if (a.r.k > 8) return false;
+    // result += is done by the store wavefronts of the plain launch where every row is written once
+    if (a.accumulate && !(a.act == HEXA_ACT_NONE && (a.out_per_slot || a.r.k == 1))) return false;
     // copies address their operands as base + 32-bit byte offset
     if ((size_t)a.r.T * (a.x_per_slot ? a.r.k : 1) * a.in_dim * 2 >= ((size_t)1 << 32) || (size_t)a.in_dim * a.out_dim * 2 >= ((size_t)1 << 32) ||
         (size_t)a.r.T * a.r.k * a.out_dim * 2 >= ((size_t)1 << 32))
@@ -659,7 +668,7 @@ int launch_esmm16_pipe(const EsmmArgs& a, hipStream_t st) {
     p.x_slot_rows = a.x_per_slot ? a.r.T : 0;
     p.out_slot_rows = a.out_per_slot ? a.r.T : 0;
     p.bias_dt = a.bias_dt; p.out_dt = a.out_dt; p.act = a.act;
-    p.stream_out = option(OPT_ESMM_STREAM) != 2; p.colsum = a.colsum; p.group = 0; p.accumulate = 0;
+    p.stream_out = option(OPT_ESMM_STREAM) != 2; p.colsum = a.colsum; p.group = 0; p.accumulate = a.accumulate;
     p.ws = (!a.out_per_slot && a.r.k > 1) ? a.slot_ws : nullptr;
     p.slot_begin = 0; p.nslots = a.r.k;
     p.total = (long)p.nslots * p.mt_ub * p.ntn;

@@ -26,6 +26,7 @@ SHAPES = [
     (1000, 384, 256, 8, 2, None),
     (700, 200, 72, 4, 1, "one"),
     (2048, 128, 512, 8, 1, None),
+    (900, 320, 136, 6, 1, None),      # one slot, a contraction the pipelined kernel takes (also when accumulating)
     (1500, 264, 392, 16, 2, "zipf"),
     (1100, 512, 384, 8, 2, None),     # a 384-wide result: one tile spans it
     (900, 96, 328, 5, 2, "zipf"),

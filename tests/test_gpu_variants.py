@@ -50,6 +50,10 @@ def test_variant(dev, knobs, cfg, dtype, dims):
     Wt = W.transpose(1, 2).contiguous().to(dev)
     got = ops.esmm(x.to(dev), Wt, b.to(dev), route, False, _lib.HEXA_W_OUT_IN)
     assert_close(got, want, TOL[dtype], "esmm out_in")
+    base = torch.randn(want.shape, generator=g).to(dtype)
+    acc = base.clone().to(dev)
+    ops.esmm(x.to(dev), Wt, b.to(dev), route, False, _lib.HEXA_W_OUT_IN, out=acc, accumulate=True)
+    assert_close(acc, want + base.float(), TOL[dtype], "esmm accumulating")
     y1r = y1.float().cpu().double().requires_grad_(True)
     lin = O.esmm(x.float(), W.float(), None, token_ids, offsets, False)
     (want_g,) = torch.autograd.grad(torch.nn.functional.gelu(y1r), y1r, lin.double())

@@ -347,9 +347,11 @@ struct Cursor {   // walks the expert's token list in 32-token steps, slot after
 
 // fp32 result rows staged per pass, and the LDS area that holds both the stages and that staging
 template <typename C> constexpr int estmm_pass_rows() {
-    // the largest multiple-of-32 divisor of BM whose staged fp32 rows fit in the stage buffers
+    // the largest multiple-of-32 divisor of BM whose staged fp32 rows fit in the stage buffers, or in 34 KB where
+    // those are smaller (64 rows of a 128-wide block: two passes instead of four for 2 KB more LDS per workgroup)
+    constexpr int room = C::STAGE_AREA > 34 * 1024 ? C::STAGE_AREA : 34 * 1024;
     for (int rows = C::BM; rows > 32; rows /= 2)
-        if (rows * (C::BN + 4) * 4 <= C::STAGE_AREA) return rows;
+        if (rows * (C::BN + 4) * 4 <= room) return rows;
     return 32;
 }
 template <typename C> constexpr int estmm_stage_area() {
@@ -643,8 +645,9 @@ int launch_estmm_dma_c(const EstmmArgs& a, hipStream_t st) {
     if (a.plan && a.scratch && a.max_slots >= 2 && (mn & 3) == 0) {
         p.plan = a.plan;
         p.scratch = a.scratch;
-        // every cut adds at most PLAN_MAX_PARTS-1 units and uses at least 2 slots
-        units = E + (int)std::min<long>((long)(a.max_slots / 2) * (PLAN_MAX_PARTS - 1), (long)E * (PLAN_MAX_PARTS - 1));
+        // a list cut into n parts adds n - 1 units and holds n >= 2 of the slots: at most max_slots - 1 more units
+        // (workgroups past the plan's unit count leave at once, but tens of thousands of them are not free)
+        units = E + (int)std::min<long>(a.max_slots - 1, (long)E * (PLAN_MAX_PARTS - 1));
     }
     p.total = (long)units * p.mtn * p.ntn;
     if (p.total == 0) return HEXA_OK;

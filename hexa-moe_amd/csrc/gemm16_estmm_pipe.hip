@@ -6,12 +6,12 @@
 //   * 4 "multiply" wavefronts (2 x 2, 64 x 64 results each): transposing LDS fragment reads and MFMAs only;
 //   * 4 "copy" wavefronts issue every asynchronous global->LDS copy: both operands are gathered by token id, 64
 //     tokens per stage, three stages deep, and the pipeline never drains between items -- the first stages of the
-//     next item are in flight while the current one finishes; the token ids travel through an LDS ring four steps
-//     ahead of the rows they address;
+//     next item are in flight while the current one finishes; the token ids travel through an LDS ring, fetched seven
+//     steps before the step they belong to;
 //   * 4 "store" wavefronts write the previous item's result (staged in LDS by the multiply wavefronts) while the
 //     next item is being multiplied;
-//   * 1 "scheduler" wavefront pops the queue a few steps ahead (one atomic per item, its latency hidden behind the
-//     steps in between) and publishes item records in LDS for the other roles.
+//   * 1 "scheduler" wavefront pops the queue up to 24 steps ahead (one atomic per batch of items, its latency hidden
+//     behind the steps in between) and publishes item records in LDS for the other roles.
 //
 // The queue is eight counters, one per XCD: the items (heaviest expert first, as the plan orders them) are dealt to
 // the XCDs in runs that share token rows, a workgroup pops its own XCD's counter and moves on to the next XCD's when
